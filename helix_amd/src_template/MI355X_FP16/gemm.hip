@@ -1,0 +1,433 @@
+// MI355X (gfx950 / CDNA4) FP16 GEMM + implicit-GEMM convolution template.
+//
+//   GEMM : C[M x N] = A[M x K] * B[N x K]^T          FP16 in, FP32 accumulate (MFMA), FP16 out
+//   CONV : y[B,OH,OW,OC] = conv2d(x[B,H,W,IC], w[OC,kH,kW,IC])  == the same GEMM with
+//          M = B*OH*OW, N = OC, K = kH*kW*IC, where the A tile is gathered from x on the fly.
+//
+// Role in the reference: this file stands where src_template/Ampere_FP16/gemm.cu (tensor-core HGEMM,
+// :120-534), gemm_splitK.cu (:120-509) and the im2col.cu + GEMM pair (im2col.cu:38-97) stand.  The
+// operand layout (B stored N x K) follows gemm.cu:144,597-601; unlike the reference's
+// `mma...f16.f16.f16.f16` (gemm.cu:54-57) accumulation is FP32.
+//
+// Compile-time parameters (set with -D by the build script, one shared library per combination):
+//   BLOCK_ROWS x BLOCK_COLS   workgroup tile of C           (reference BLOCK_ROWS / BLOCK_COLS)
+//   WAVE_ROWS  x WAVE_COLS    tile of C owned by one wave64 (reference WARP_ROWS / WARP_COLS)
+//   BLOCK_K                   K extent of one LDS stage
+//   LDS_STAGES                LDS ring depth                (reference K_STAGE)
+//   SPLIT_K                   K partitions (FP32 workspace + reduction kernel when > 1)
+//
+// Kernel structure
+//   * one wave64 computes (WAVE_ROWS/32) x (WAVE_COLS/32) v_mfma_f32_32x32x16_f16 tiles; per 16-wide
+//     k step it reads one 16-byte fragment per 32 rows of A and of B from LDS (ds_read_b128).
+//   * global -> LDS goes through buffer loads (128-bit per lane, hardware bounds checking zero-fills
+//     rows beyond M / N) into registers and ds_write_b128; the loads for stage s+1 are issued before
+//     the MFMAs of stage s and written to LDS after them, one barrier per stage.
+//   * LDS rows are BLOCK_K halves; 16-byte chunk c of row r is stored at chunk (c ^ key(r)), with
+//     key(r) = (r / rows_per_256B) mod chunks_per_row, so that 16 consecutive rows of one chunk column
+//     land in 16 different 16-byte bank groups (64 banks x 4 B): fragment reads and tile writes are
+//     both conflict-free.
+//   * workgroup id -> tile: ids are dealt round-robin to the 8 XCDs by the hardware, so id is first
+//     remapped to (xcd, slot) -> xcd * ids_per_xcd + slot, then walked in column-major groups of
+//     GROUP_ROWS tile rows; each XCD's L2 then sees a compact patch of tiles sharing A and B panels.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../../include/helix_abi.h"
+
+#ifndef BLOCK_ROWS
+#define BLOCK_ROWS 256
+#endif
+#ifndef BLOCK_COLS
+#define BLOCK_COLS 256
+#endif
+#ifndef WAVE_ROWS
+#define WAVE_ROWS 128
+#endif
+#ifndef WAVE_COLS
+#define WAVE_COLS 128
+#endif
+#ifndef BLOCK_K
+#define BLOCK_K 64
+#endif
+#ifndef LDS_STAGES
+#define LDS_STAGES 2
+#endif
+#ifndef SPLIT_K
+#define SPLIT_K 1
+#endif
+#ifndef GROUP_ROWS
+#define GROUP_ROWS 8
+#endif
+
+namespace {
+
+typedef _Float16 half_t;
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+
+constexpr int BM = BLOCK_ROWS, BN = BLOCK_COLS, WM = WAVE_ROWS, WN = WAVE_COLS, BK = BLOCK_K;
+constexpr int STAGES = LDS_STAGES, SPLITK = SPLIT_K;
+constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN, NWAVES = WAVES_M * WAVES_N, NTHREADS = 64 * NWAVES;
+constexpr int TM = WM / 32, TN = WN / 32;      // MFMA tiles per wave
+constexpr int KCH = BK / 8;                    // 16-byte chunks per LDS row
+constexpr int ROW_BYTES = BK * 2;
+constexpr int RP = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;  // rows per 256 bytes of LDS
+constexpr int A_ITERS = BM * KCH / NTHREADS, B_ITERS = BN * KCH / NTHREADS;
+constexpr int ROWS_PER_ITER = NTHREADS / KCH;
+constexpr int A_STAGE_BYTES = BM * ROW_BYTES, B_STAGE_BYTES = BN * ROW_BYTES;
+constexpr int STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
+constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+
+static_assert(BM % WM == 0 && BN % WN == 0, "block tile must be a multiple of the wave tile");
+static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is built from 32x32 MFMA tiles");
+static_assert(BK % 16 == 0 && (KCH & (KCH - 1)) == 0 && KCH >= 2, "BLOCK_K must be 16 * 2^n");
+static_assert(NTHREADS <= 1024 && NTHREADS % KCH == 0, "bad thread count");
+static_assert((BM * KCH) % NTHREADS == 0 && (BN * KCH) % NTHREADS == 0, "tile copy must divide evenly");
+static_assert(STAGES == 2, "this revision implements the two-stage ring");
+static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
+static_assert(SPLITK >= 1 && SPLITK <= 8, "SPLIT_K out of range");
+
+struct ConvGeom {
+    int H, W, IC, OH, OW, kW, stride, pad, M;  // M = batch*OH*OW
+};
+
+struct Params {
+    const half_t* A;   // GEMM: M x K (lda).  CONV: x, NHWC
+    const half_t* B;   // N x K (ldb).        CONV: w, [OC][kH][kW][IC]
+    half_t* C;         // M x N (ldc)
+    float* ws;         // SPLIT_K > 1: [SPLIT_K][M][N] FP32 partial sums
+    int M, N, K, lda, ldb, ldc;
+    int tiles_m, tiles_n;
+    unsigned a_bytes;  // CONV: size of x in bytes (bounds for the gather)
+    ConvGeom g;
+};
+
+__device__ __forceinline__ int swz_key(int row) { return (row / RP) & (KCH - 1); }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ intx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) {
+    return __builtin_bit_cast(intx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+}
+
+template <bool CONV>
+__global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+
+    // ---- workgroup id -> (tile_m, tile_n), XCD-aware ------------------------------------------
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = ntiles / 8, rem = ntiles % 8;
+        const int xcd = pid % 8, slot = pid / 8;
+        pid = xcd * per + (xcd < rem ? xcd : rem) + slot;
+    }
+    const int group_tiles = GROUP_ROWS * p.tiles_n;
+    const int grp = pid / group_tiles;
+    const int first_m = grp * GROUP_ROWS;
+    const int gsize = (p.tiles_m - first_m) < GROUP_ROWS ? (p.tiles_m - first_m) : GROUP_ROWS;
+    const int in_grp = pid % group_tiles;
+    const int tile_m = first_m + in_grp % gsize;
+    const int tile_n = in_grp / gsize;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    // ---- K range of this workgroup (split-K partitions are multiples of BLOCK_K) -----------------
+    int k_begin = 0, k_end = p.K;
+    if (SPLITK > 1) {
+        const int ktiles = (p.K + BK - 1) / BK;
+        const int per = (ktiles + SPLITK - 1) / SPLITK;
+        k_begin = (int)blockIdx.y * per * BK;
+        k_end = k_begin + per * BK;
+        if (k_end > p.K) k_end = p.K;
+        if (k_begin > p.K) k_begin = p.K;
+    }
+
+    // ---- per-thread copy geometry ---------------------------------------------------------------
+    const int kc = tid % KCH;          // 16-byte chunk within a tile row (same for every iteration)
+    const int r0 = tid / KCH;          // first tile row this thread copies
+    int lds_wr_a[A_ITERS], lds_wr_b[B_ITERS];
+#pragma unroll
+    for (int i = 0; i < A_ITERS; i++) {
+        const int r = r0 + i * ROWS_PER_ITER;
+        lds_wr_a[i] = r * ROW_BYTES + ((kc ^ swz_key(r)) << 4);
+    }
+#pragma unroll
+    for (int i = 0; i < B_ITERS; i++) {
+        const int r = r0 + i * ROWS_PER_ITER;
+        lds_wr_b[i] = A_STAGE_BYTES + r * ROW_BYTES + ((kc ^ swz_key(r)) << 4);
+    }
+
+    // B operand: rows n0.. of an N x K matrix
+    const int rows_b = (p.N - n0) < BN ? (p.N - n0) : BN;
+    const half_t* baseB = p.B + (size_t)n0 * p.ldb;
+    const unsigned bytesB = (unsigned)(((size_t)(rows_b - 1) * p.ldb + p.K) * 2);
+    int voff_b[B_ITERS];
+#pragma unroll
+    for (int i = 0; i < B_ITERS; i++) voff_b[i] = ((r0 + i * ROWS_PER_ITER) * p.ldb + kc * 8) * 2;
+
+    // A operand
+    const half_t* baseA = nullptr;
+    unsigned bytesA = 0;
+    int voff_a[A_ITERS];
+    int cv_img[A_ITERS], cv_ih[A_ITERS], cv_iw[A_ITERS];  // CONV: image base offset, top-left tap coords
+    if (!CONV) {
+        const int rows_a = (p.M - m0) < BM ? (p.M - m0) : BM;
+        baseA = p.A + (size_t)m0 * p.lda;
+        bytesA = (unsigned)(((size_t)(rows_a - 1) * p.lda + p.K) * 2);
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) voff_a[i] = ((r0 + i * ROWS_PER_ITER) * p.lda + kc * 8) * 2;
+    } else {
+        baseA = p.A;
+        bytesA = p.a_bytes;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) {
+            const int m = m0 + r0 + i * ROWS_PER_ITER;
+            const int ow = m % p.g.OW;
+            const int t = m / p.g.OW;
+            const int oh = t % p.g.OH;
+            const int b = t / p.g.OH;
+            cv_img[i] = (m < p.g.M) ? b * p.g.H * p.g.W : -1;
+            cv_ih[i] = oh * p.g.stride - p.g.pad;
+            cv_iw[i] = ow * p.g.stride - p.g.pad;
+        }
+    }
+
+    intx4 stage_a[A_ITERS], stage_b[B_ITERS];
+
+    auto load_global = [&](int k0) {
+        const bool tail = (k0 + BK > p.K);
+        const bool dead = tail && (k0 + kc * 8 >= p.K);  // chunk lies beyond K: contributes zero
+        __amdgpu_buffer_rsrc_t rb = make_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u);
+#pragma unroll
+        for (int i = 0; i < B_ITERS; i++) {
+            stage_b[i] = buf_load16(rb, dead ? (int)0x7fffffff : voff_b[i]);
+        }
+        if (!CONV) {
+            __amdgpu_buffer_rsrc_t ra = make_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
+#pragma unroll
+            for (int i = 0; i < A_ITERS; i++) {
+                stage_a[i] = buf_load16(ra, dead ? (int)0x7fffffff : voff_a[i]);
+            }
+        } else {
+            __amdgpu_buffer_rsrc_t ra = make_rsrc(baseA, bytesA);
+            const int k = k0 + kc * 8;       // k = (kh*kW + kw)*IC + c, 8 consecutive c per chunk
+            const int c = k % p.g.IC;
+            const int t = k / p.g.IC;
+            const int kw = t % p.g.kW;
+            const int kh = t / p.g.kW;
+#pragma unroll
+            for (int i = 0; i < A_ITERS; i++) {
+                const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
+                const bool ok = !dead && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W;
+                const int off = ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 2;
+                stage_a[i] = buf_load16(ra, ok ? off : (int)0x7fffffff);
+            }
+        }
+    };
+
+    auto store_lds = [&](int stage) {
+        unsigned char* base = smem + stage * STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) *(intx4*)(base + lds_wr_a[i]) = stage_a[i];
+#pragma unroll
+        for (int i = 0; i < B_ITERS; i++) *(intx4*)(base + lds_wr_b[i]) = stage_b[i];
+    };
+
+    // ---- fragment read geometry -----------------------------------------------------------------
+    // MFMA 32x32x16: lane l supplies row (l % 32), k = 8*(l/32) .. +7 of both operands.
+    const int frow = lane & 31, fhalf = lane >> 5;
+    const int a_row = wave_m * WM + frow;
+    const int b_row = wave_n * WN + frow;
+    const int a_rd = a_row * ROW_BYTES, b_rd = A_STAGE_BYTES + b_row * ROW_BYTES;
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    const int ktiles = (k_end - k_begin + BK - 1) / BK;
+    if (ktiles > 0) {
+        load_global(k_begin);
+        store_lds(0);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < ktiles; kt++) {
+        const int cur = kt & 1;
+        const bool more = (kt + 1 < ktiles);
+        if (more) load_global(k_begin + (kt + 1) * BK);
+
+        const unsigned char* sb = smem + cur * STAGE_BYTES;
+#pragma unroll
+        for (int s = 0; s < BK / 16; s++) {
+            half8 af[TM], bf[TN];
+            const int ch = s * 2 + fhalf;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                af[i] = *(const half8*)(sb + a_rd + i * 32 * ROW_BYTES + ((ch ^ swz_key(a_row + i * 32)) << 4));
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                bf[j] = *(const half8*)(sb + b_rd + j * 32 * ROW_BYTES + ((ch ^ swz_key(b_row + j * 32)) << 4));
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+
+        if (more) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane l holds column (l % 32); rows 8*(v/4) + 4*(l/32) + (v%4), v = 0..15 -------
+    const int col_l = lane & 31, row_l = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = n0 + wave_n * WN + j * 32 + col_l;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wave_m * WM + i * 32 + (v / 4) * 8 + row_l + (v % 4);
+                if (row < p.M && col < p.N) {
+                    if (SPLITK > 1)
+                        p.ws[((size_t)blockIdx.y * p.M + row) * p.N + col] = acc[i][j][v];
+                    else
+                        p.C[(size_t)row * p.ldc + col] = (half_t)acc[i][j][v];
+                }
+            }
+        }
+    }
+}
+
+// Sums the SPLIT_K FP32 partials in a fixed order and rounds once to FP16 (deterministic, unlike
+// the reference's half2 atomics, src_template/Ampere_FP16/gemm_splitK.cu:495-506).
+__global__ void helix_splitk_reduce_kernel(const float* ws, half_t* C, int M, int N, int ldc, int splits) {
+    const size_t total = (size_t)M * N;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        float s = 0.f;
+        for (int k = 0; k < splits; k++) s += ws[(size_t)k * total + idx];
+        const size_t row = idx / N, col = idx % N;
+        C[row * ldc + col] = (half_t)s;
+    }
+}
+
+}  // namespace
+
+// -------------------------------------------------------------------------------------------------
+// host side
+// -------------------------------------------------------------------------------------------------
+#include <stdio.h>
+
+namespace tpl {
+
+constexpr int kElemBytes = 2;
+
+inline const char* info_json() {
+    static char buf[1024];
+    static bool done = false;
+    if (!done) {
+        snprintf(buf, sizeof(buf),
+                 "{\"family\": \"gemm_f16\", \"arch\": \"gfx950\", \"mfma\": \"v_mfma_f32_32x32x16_f16\", "
+                 "\"lds_stages\": %d, \"block_rows\": %d, \"block_cols\": %d, \"wave_rows\": %d, \"wave_cols\": %d, "
+                 "\"block_k\": %d, \"split_k\": %d, \"threads\": %d, \"lds_bytes\": %d, "
+                 "\"layout_a\": \"M x K row-major f16\", \"layout_b\": \"N x K row-major f16\", "
+                 "\"layout_c\": \"M x N row-major f16\", \"accumulate\": \"f32\", "
+                 "\"k_multiple\": 8, \"ld_multiple\": 8, \"conv\": \"NHWC x [OC][kH][kW][IC], IC %% 8 == 0\"}",
+                 STAGES, BM, BN, WM, WN, BK, SPLITK, NTHREADS, LDS_BYTES);
+        done = true;
+    }
+    return buf;
+}
+
+inline size_t workspace_bytes(int M, int N, int K) {
+    (void)K;
+    return SPLITK > 1 ? (size_t)SPLITK * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
+inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce, int* lda, int* ldb, int* ldc) {
+    *ae = (size_t)M * K; *be = (size_t)N * K; *ce = (size_t)M * N;
+    *lda = K; *ldb = K; *ldc = N;
+}
+
+template <bool CONV>
+inline int set_lds_attr() {
+    static int rc = (int)hipFuncSetAttribute((const void*)helix_gemm_f16_kernel<CONV>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    return rc;
+}
+
+template <bool CONV>
+inline int launch(const Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (SPLITK > 1) {
+        const size_t need = workspace_bytes(p.M, p.N, p.K);
+        if (!ws || ws_bytes < need) return HELIX_ERR_WORKSPACE;
+    }
+    int rc = set_lds_attr<CONV>();
+    if (rc) return rc;
+    const long long ntiles = (long long)p.tiles_m * p.tiles_n;
+    if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    dim3 grid((unsigned)ntiles, SPLITK, 1), block(NTHREADS, 1, 1);
+    hipLaunchKernelGGL(helix_gemm_f16_kernel<CONV>, grid, block, LDS_BYTES, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    if (SPLITK > 1) {
+        size_t total = (size_t)p.M * p.N;
+        int blocks = (int)((total + 255) / 256);
+        if (blocks > 8192) blocks = 8192;
+        hipLaunchKernelGGL(helix_splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, (const float*)ws, p.C, p.M,
+                           p.N, p.ldc, SPLITK);
+        e = hipGetLastError();
+        if (e != hipSuccess) return (int)e;
+    }
+    return 0;
+}
+
+inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc, void* ws,
+                size_t ws_bytes, hipStream_t s) {
+    if (K % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0) return HELIX_ERR_INVALID_VALUE;
+    if (lda < K || ldb < K || ldc < N) return HELIX_ERR_INVALID_VALUE;
+    if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)C & 1)) return HELIX_ERR_INVALID_VALUE;
+    // per-tile byte offsets are 32-bit
+    if ((long long)BM * lda * 2 >= 0x7fffffffLL || (long long)BN * ldb * 2 >= 0x7fffffffLL)
+        return HELIX_ERR_INVALID_VALUE;
+    Params p{};
+    p.A = (const half_t*)A; p.B = (const half_t*)B; p.C = (half_t*)C; p.ws = (float*)ws;
+    p.M = M; p.N = N; p.K = K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    p.tiles_m = (M + BM - 1) / BM; p.tiles_n = (N + BN - 1) / BN;
+    return launch<false>(p, ws, ws_bytes, s);
+}
+
+inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
+                  int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (IC % 8 != 0) return HELIX_ERR_INVALID_VALUE;  // a 16-byte chunk must stay inside one filter tap
+    const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
+    const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
+    const long long xbytes = (long long)batch * H * W * IC * 2;
+    if (M > 0x7fffffffLL || K > 0x7fffffffLL || xbytes >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    if ((long long)BN * K * 2 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 1)) return HELIX_ERR_INVALID_VALUE;
+    Params p{};
+    p.A = (const half_t*)x; p.B = (const half_t*)w; p.C = (half_t*)y; p.ws = (float*)ws;
+    p.M = (int)M; p.N = OC; p.K = (int)K; p.lda = 0; p.ldb = (int)K; p.ldc = OC;
+    p.tiles_m = (int)((M + BM - 1) / BM); p.tiles_n = (OC + BN - 1) / BN;
+    p.a_bytes = (unsigned)xbytes;
+    p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M};
+    return launch<true>(p, ws, ws_bytes, s);
+}
+
+}  // namespace tpl
+
+#include "../common/helix_host.h"
