@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Headline benchmark: autotuned FP16 GEMM (FP16 in, FP32 accumulate, FP16 out) at M=N=K=8192 on one
+MI355X, reported as TFLOP/s and as a fraction of the FP16 MFMA peak, with the decode-GEMV HBM rate,
+the autotune wall time and the CPU baseline (the restated x86_CPU path on the host cores) beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one GEMM launch through the C ABI (helix_gemm) on operands already resident in HBM.  Prints
+one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "helix_amd", "scripts"))
+os.chdir(ROOT)
+
+SIZE = 8192
+
+
+def autotune(prof_keys, M, N, K):
+    """Full template search for one shape: run every MFMA configuration, keep the fastest."""
+    from MI355X_FP16.MI355X_FP16_gemm import run_config
+    best, best_t, tried = None, float("inf"), 0
+    for k in prof_keys:
+        if k[0] == 0:
+            continue
+        try:
+            t = run_config(k, M, N, K, warmup=1, iters=3)
+        except Exception:
+            continue
+        tried += 1
+        if t < best_t:
+            best, best_t = k, t
+    if best is None:
+        raise RuntimeError("no MI355X_FP16 kernel library could run; build them with __graft_entry__.build()")
+    return best, best_t, tried
+
+
+def gemv_rates(rotate_bytes=1 << 30):
+    """Config 3: decode GEMV, cold (weights rotated through >= 1 GiB so the 256 MB last-level cache
+    cannot hold them).  Returns a list of dicts with achieved GB/s on the algorithmic bytes."""
+    from utils.helix_runtime import load
+    from utils.roofline import gemm_bytes, HBM_BYTES_PER_S
+    from utils.get_benchmark_shape_list import BASELINE_GEMV_BATCHES, BASELINE_GEMV_KN
+    from MI355X_FP16.build_MI355X_FP16 import kernel_library
+    lib = load(kernel_library("gemv"))
+    out = []
+    for (K, N) in BASELINE_GEMV_KN:
+        for M in BASELINE_GEMV_BATCHES:
+            mn, avg, _ = lib.bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)
+            nbytes = gemm_bytes(M, N, K, 2)
+            out.append({"M": M, "K": K, "N": N, "us": round(mn * 1e6, 2), "GB/s": round(nbytes / mn / 1e9, 1),
+                        "frac_hbm_peak": round(nbytes / mn / HBM_BYTES_PER_S, 4)})
+    return out
+
+
+def cpu_baseline(budget_s=20.0):
+    """The reference's x86_CPU path (restated in oracle/) on this machine's host cores: two-phase
+    profile, tiling pick, then the packed / n-parallel schedule on a bounded FP32 GEMM sample."""
+    from oracle import oracle as O
+    cores = os.cpu_count() or 1
+    t0 = time.perf_counter()
+    _, cache = O.x86_profile(peak_gflops=None, number=200)
+    prof_s = time.perf_counter() - t0
+    s = 2048
+    # one run to size `number` so the whole leg stays near the budget
+    cost, gflops, padded, tiling, _ = O.x86_time_gemm(cache, s, s, s, num_thread=cores, number=1)
+    number = max(1, min(100, int((budget_s - prof_s) / max(cost, 1e-3))))
+    cost, gflops, padded, tiling, _ = O.x86_time_gemm(cache, s, s, s, num_thread=cores, number=number)
+    return {"value": round(gflops / 1e3, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"FP32 GEMM {s}^3 (padded to {padded[0]}x{padded[1]}x{padded[2]}), restated x86_CPU schedule "
+                      f"tiling {tiling}, mean of {number} runs; x86 profile took {prof_s:.1f} s",
+            "isa": O.isa()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gemv", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (every GPU box has one GPU); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from utils import seeded_inputs
+    from utils.helix_runtime import load
+    from utils.roofline import FP16_MFMA_FLOPS, gemm_flops
+    from MI355X_FP16.build_MI355X_FP16 import library_for_key
+    from MI355X_FP16.profile_MI355X_FP16 import all_keys
+
+    if not torch.cuda.is_available():
+        raise RuntimeError("bench.py needs an MI355X; there is no CPU fallback for the HIP path")
+    dev = torch.device("cuda:0")
+    M = N = K = SIZE
+
+    # ---- autotune: full template search on this shape ------------------------------------------------
+    t0 = time.perf_counter()
+    best, best_t, tried = autotune(all_keys(), M, N, K)
+    autotune_s = time.perf_counter() - t0
+    lib = load(library_for_key(best))
+
+    # ---- seeded operands, resident in HBM before the timed region --------------------------------------
+    A_h, B_h = seeded_inputs.gemm_operands(M, N, K, np.float16)          # A (M,K), B (K,N)
+    A = torch.from_numpy(A_h).to(dev)
+    Bt = torch.from_numpy(np.ascontiguousarray(B_h.T)).to(dev)           # device layout: N x K
+    C = torch.empty((M, N), dtype=torch.float16, device=dev)
+    wsb = lib.workspace_bytes(M, N, K)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        lib.gemm(A.data_ptr(), Bt.data_ptr(), C.data_ptr(), M, N, K, K, K, N, ws.data_ptr(), wsb, stream)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed / args.steps * 1e3
+    flops = gemm_flops(M, N, K)
+    value = flops / (elapsed / args.steps) / 1e12
+
+    # ---- dominant kernel, HIP events on the launch stream -----------------------------------------------
+    kern_s = lib.gemm_timed(A.data_ptr(), Bt.data_ptr(), C.data_ptr(), M, N, K, K, K, N, ws.data_ptr(), wsb, stream,
+                            warmup=2, iters=args.steps)
+    achieved = flops / kern_s / 1e12
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP16_MFMA_FLOPS / 1e12, "unit": "TFLOP/s",
+                "frac": round(achieved * 1e12 / FP16_MFMA_FLOPS, 4), "traffic": None,
+                "kernel": "helix_gemm_f16_kernel<false>", "kernel_avg_us": round(kern_s * 1e6, 2)}
+
+    # ---- spot check of the timed result against torch's FP32 matmul on a slice ------------------------------
+    ref = A[:256].float() @ Bt[:256].float().t()
+    err = (C[:256, :256].float() - ref).abs().max().item() / ref.abs().max().item()
+    if not err < 2e-2:
+        raise RuntimeError(f"timed GEMM result is wrong: normwise error {err}")
+
+    out = {
+        "metric": "FP16 GEMM TFLOP/s (autotuned, FP16 in / FP32 accumulate / FP16 out)",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16 (f32 accumulate)", "data": "synthetic",
+        "config": {"workload": f"FP16 GEMM M=N=K={SIZE}, A,B ~ N(0,0.1^2) seeded, full template search",
+                   "kernel_config": list(best), "library": os.path.basename(library_for_key(best))},
+        "pct_mfma_peak": round(100.0 * value * 1e12 / FP16_MFMA_FLOPS, 2),
+        "autotune_wall_s": round(autotune_s, 2), "autotune_candidates": tried,
+        "roofline": roofline,
+    }
+    if not args.no_gemv:
+        out["gemv_hbm"] = gemv_rates()
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,93 @@
+"""Cost model and single-GEMM runner of the MI355X_FP16 backend.
+
+Mirrors scripts/Ampere_FP16/Ampere_FP16_gemm.py:420-446 (`cost_model`, `get_Ampere_FP16_gemm_Helix_result`)
+and :548-553 (vendor-library result).  The TVM-on-GPU alternative backend of the reference (:17-417)
+has no counterpart: the only backend value is "hip".
+"""
+import math
+import os
+
+from utils.helix_runtime import load
+from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
+from MI355X_FP16.build_MI355X_FP16 import library_for_key
+from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K
+
+root_path = os.getcwd()
+
+HBM_SUSTAINED_FRACTION = 0.6  # share of the datasheet HBM rate a streaming kernel sustains
+GEMV_LAUNCH_FLOOR_S = 3e-6   # a kernel launch on an idle queue; keeps tiny problems from looking free
+
+
+def config_cost(k, v, M, N, K):
+    """Predicted seconds of configuration k (profiled round time v) on an M x N x K problem.
+
+    Reference form (Ampere_FP16_gemm.py:424-426): rounds = ceil(blocks / SMs), cost = rounds * v with
+    108 SMs and K ignored.  Here SMs -> 256 compute units and the round time is scaled by K / K_profile
+    (a round's time is proportional to the K extent each tile walks; split-K halves it)."""
+    if k[0] == 0:
+        # weight-streaming kernel: HBM-bound, so a partial round costs its share of a round (no
+        # quantisation), never less than a launch; the streamed operand is the larger of M and N
+        small, big = (M, N) if M <= N else (N, M)
+        num_block = math.ceil(small / k[1]) * math.ceil(big / k[2])
+        return max(num_block / NUM_CU * v * max(K, 512) / PROFILE_K, GEMV_LAUNCH_FLOOR_S)
+    num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * (k[5] + 1)
+    w = math.ceil(num_block / NUM_CU)
+    k_scale = max(K, 64) / PROFILE_K
+    if k[5] == 1:
+        k_scale = k_scale / 2 + 64 / PROFILE_K
+    # a tile round cannot beat streaming every operand once from HBM at the sustained rate
+    return max(w * v * k_scale, gemm_bytes(M, N, K, 2) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
+
+
+def cost_model(prof_dict, M, N, K):
+    min_cost = float("inf")
+    best_config = (1, 1, 1, 1, 1, 0, 32)
+    for k, v in prof_dict.items():
+        cost = config_cost(k, v, M, N, K)
+        if min_cost > cost:
+            min_cost = cost
+            best_config = k
+    return best_config
+
+
+def padded_k(K):
+    """The FP16 kernels load 16-byte chunks along K; a K that is not a multiple of 8 halves is run on
+    buffers whose rows are zero-padded to the next multiple (zeros add nothing to the dot products)."""
+    return math.ceil(K / 8) * 8
+
+
+def run_config(k, M, N, K, warmup=10, iters=10, outer=1):
+    """Seconds per launch (mean) of configuration k on the real, unpadded M and N.  The reference pads
+    M and N up to the tile (Ampere_FP16_gemm.py:438) because its kernel has no bounds checks; the
+    MI355X kernels predicate their edges instead."""
+    lib = load(library_for_key(k))
+    if k[0] == 0 and M > N:
+        M, N = N, M   # the GEMV kernel streams its second operand; gemv.cu:384-386 swaps the same way
+    _, avg, _ = lib.bench(M, N, padded_k(K), warmup=warmup, iters=iters, outer=outer, rotate_bytes=0)
+    return avg
+
+
+def get_MI355X_FP16_gemm_Helix_result(prof_dict, M, N, K, backend="hip"):
+    if backend != "hip":
+        raise ValueError(f"backend {backend!r} is not available for MI355X_FP16 (only 'hip')")
+    best_config = cost_model(prof_dict, M, N, K)
+    cost = run_config(best_config, M, N, K) * 1e3
+    tflops = 2 * M * N * K / 1e9 / cost
+
+    return cost, tflops
+
+
+def get_MI355X_FP16_gemm_Oracle_result(prof_dict, M, N, K):
+    """Exhaustive per-shape search: run every candidate, keep the fastest
+    (benchmark_Ampere_FP16_performance_comparison.py:56-69).  Returns (cost_ms, tflops, key)."""
+    min_cost, best = float("inf"), None
+    for k in prof_dict.keys():
+        if k[0] == 0 and min(M, N) > 16:
+            continue   # the weight-streaming kernel re-reads the weights per 16 activation rows
+        try:
+            cost = run_config(k, M, N, K, warmup=2, iters=5)
+        except Exception:
+            continue
+        if min_cost > cost:
+            min_cost, best = cost, k
+    return min_cost * 1e3, 2 * M * N * K / 1e12 / min_cost, best

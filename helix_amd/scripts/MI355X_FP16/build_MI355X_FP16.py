@@ -1,0 +1,142 @@
+"""Build step of the MI355X_FP16 backend: instantiate the tile / wave / LDS parameter space of the
+FP16 templates and compile every point with hipcc into its own shared library.
+
+Mirrors scripts/Ampere_FP16/build_Ampere_FP16.py (compile_kernel :7-28, is_valid_config :30-39, the
+five nested loops :47-53, the fixed kernels gemv / gemv_splitK :62-65) with the same entry-point
+names modulo the backend tag.  Differences that follow from the target:
+  * output is build/bin_fp16/lib<kernel>_<params>.so exporting the C ABI of include/helix_abi.h instead of
+    an executable; the convolution path lives in the same library as the GEMM of each configuration
+    (implicit GEMM), so there is no im2col artifact;
+  * wave tiles are multiples of the 32x32 MFMA tile, K_STAGE becomes LDS_STAGES, and BLOCK_K is a
+    template parameter too (it is fixed to 32 in the reference, gemm.cu:77);
+  * compiles run in parallel worker threads instead of one os.system at a time.
+"""
+import os
+from tqdm import tqdm
+
+from utils.helix_runtime import SRC_ROOT, bin_dir, compile_many
+
+root_path = os.getcwd()
+
+LDS_STAGES_LIST = [2]
+WAVE_TILE_LIST = [32, 64, 128]
+BLOCK_SCALE_LIST = [1, 2, 4]
+BLOCK_K_LIST = [32, 64]
+LDS_LIMIT = 160 * 1024
+
+
+def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, wave_rows, wave_cols,
+                    block_k=64, lds_stages=2):
+    # the reference's four rules (build_Ampere_FP16.py:30-39)
+    if block_rows_scale == 4 and block_cols_scale == 4:
+        return False
+    if block_rows > 256 or block_cols > 256:
+        return False
+    if wave_cols == wave_rows * 8 or wave_rows == wave_cols * 8:
+        return False
+    if block_cols == block_rows * 16 or block_rows == block_cols * 16:
+        return False
+    # gfx950 resources: LDS ring, FP32 accumulators per lane, even split of the tile copy over threads
+    if lds_stages * (block_rows + block_cols) * block_k * 2 > LDS_LIMIT:
+        return False
+    if wave_rows * wave_cols // 64 > 256:
+        return False
+    threads = 64 * block_rows_scale * block_cols_scale
+    chunks_per_row = block_k // 8
+    if (block_rows * chunks_per_row) % threads or (block_cols * chunks_per_row) % threads:
+        return False
+    if threads % chunks_per_row:
+        return False
+    return True
+
+
+def iter_configs():
+    """Yields (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in build order."""
+    for LDS_STAGES in LDS_STAGES_LIST:
+        for WAVE_ROWS in WAVE_TILE_LIST:
+            for WAVE_COLS in WAVE_TILE_LIST:
+                for BLOCK_ROWS_SCALE in BLOCK_SCALE_LIST:
+                    for BLOCK_COLS_SCALE in BLOCK_SCALE_LIST:
+                        for BLOCK_K in BLOCK_K_LIST:
+                            BLOCK_ROWS = BLOCK_ROWS_SCALE * WAVE_ROWS
+                            BLOCK_COLS = BLOCK_COLS_SCALE * WAVE_COLS
+                            if not is_valid_config(BLOCK_ROWS_SCALE, BLOCK_COLS_SCALE, BLOCK_ROWS, BLOCK_COLS,
+                                                   WAVE_ROWS, WAVE_COLS, BLOCK_K, LDS_STAGES):
+                                continue
+                            yield (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K)
+
+
+def kernel_library(kernel_name, lds_stages=None, block_rows=None, block_cols=None, wave_rows=None, wave_cols=None,
+                   block_k=None):
+    """Path of the shared library of one configuration (same naming scheme as the reference's
+    executables, build_Ampere_FP16.py:13-27, plus the BLOCK_K field)."""
+    output_name = kernel_name
+    for v in (lds_stages, block_rows, block_cols, wave_rows, wave_cols, block_k):
+        if v is not None:
+            output_name += f"_{v}"
+    return f"{bin_dir('fp16')}/lib{output_name}.so"
+
+
+def library_for_key(key):
+    """prof-dict key -> library path.  key = (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS,
+    splitK flag, BLOCK_K); key[0] == 0 marks the GEMV kernels, as in the reference
+    (scripts/Ampere_FP16/Ampere_FP16_gemm.py:435)."""
+    if key[0] == 0:
+        return kernel_library("gemv" if key[5] == 0 else "gemv_splitK")
+    return kernel_library("gemm" if key[5] == 0 else "gemm_splitK", key[0], key[1], key[2], key[3], key[4], key[6])
+
+
+def compile_job(kernel_name, lds_stages=None, block_rows=None, block_cols=None, wave_rows=None, wave_cols=None,
+                block_k=None):
+    defines = {}
+    src_name = kernel_name
+    if kernel_name == "gemm_splitK":
+        src_name = "gemm"
+        defines["SPLIT_K"] = 2
+    elif kernel_name == "gemv_splitK":
+        src_name = "gemv"
+        defines["SPLIT_K"] = 4
+    if lds_stages is not None:
+        defines["LDS_STAGES"] = lds_stages
+    if block_rows is not None:
+        defines["BLOCK_ROWS"] = block_rows
+    if block_cols is not None:
+        defines["BLOCK_COLS"] = block_cols
+    if wave_rows is not None:
+        defines["WAVE_ROWS"] = wave_rows
+    if wave_cols is not None:
+        defines["WAVE_COLS"] = wave_cols
+    if block_k is not None:
+        defines["BLOCK_K"] = block_k
+    src = f"{SRC_ROOT}/MI355X_FP16/{src_name}.hip"
+    out = kernel_library(kernel_name, lds_stages, block_rows, block_cols, wave_rows, wave_cols, block_k)
+    return (src, out, defines)
+
+
+def build_jobs():
+    jobs = []
+    for cfg in iter_configs():
+        jobs.append(compile_job("gemm", *cfg))
+        jobs.append(compile_job("gemm_splitK", *cfg))
+    jobs.append(compile_job("gemv"))
+    jobs.append(compile_job("gemv_splitK"))
+    return jobs
+
+
+def build_Helix_MI355X_FP16_gemm_kernel():
+    if not os.path.exists(f"{root_path}/build/bin_fp16"):
+        os.makedirs(f"{root_path}/build/bin_fp16")
+
+    print("Start building MI355X FP16 GEMM kernel ...")
+    jobs = build_jobs()
+    with tqdm(total=len(jobs), desc="building") as pbar:
+        failed = compile_many(jobs, progress=pbar)
+    for out, err in failed:
+        print(f"Build failed: {out}\n{err}")
+    print("Build finished.")
+    return failed
+
+
+if __name__ == "__main__":
+
+    build_Helix_MI355X_FP16_gemm_kernel()

@@ -1,0 +1,40 @@
+"""Convolution runner of the MI355X_FP32 backend (implicit GEMM, NHWC, FP32).
+Mirrors scripts/Ampere_FP32/Ampere_FP32_conv.py:89-110; one kernel instead of im2col + SGEMM (the
+reference even borrows the FP16 im2col binary here, :107)."""
+import math
+import os
+
+from utils.helix_runtime import load
+from MI355X_FP32.build_MI355X_FP32 import library_for_key
+from MI355X_FP32.MI355X_FP32_gemm import config_cost
+
+root_path = os.getcwd()
+
+
+def cost_model(prof_dict, M, N, K):
+    min_cost = float("inf")
+    best_config = (1, 1, 1, 1, 1, 1, 1, 1)
+    for k, v in prof_dict.items():
+        if k[2] == 0:
+            continue
+        cost = config_cost(k, v, M, N, K)
+        if min_cost > cost:
+            min_cost = cost
+            best_config = k
+    return best_config
+
+
+def get_MI355X_FP32_conv_Helix_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
+                                      backend="hip"):
+    if backend != "hip":
+        raise ValueError(f"backend {backend!r} is not available for MI355X_FP32 (only 'hip')")
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    N = output_channel
+    K = input_channel * kH * kW
+    best_config = cost_model(prof_dict, M, N, K)
+    lib = load(library_for_key(best_config))
+    _, avg, _ = lib.bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad, warmup=10, iters=10)
+    cost = avg * 1e3
+    tflops = 2 * M * N * K / 1e9 / cost
+
+    return cost, tflops

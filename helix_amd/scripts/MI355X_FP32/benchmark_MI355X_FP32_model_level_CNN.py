@@ -1,0 +1,37 @@
+"""Model-level CNN benchmark of the MI355X_FP32 backend: summed per-layer latency.
+Mirrors scripts/Ampere_FP32/benchmark_Ampere_FP32_model_level_CNN.py:9-27."""
+import math
+import os
+
+from utils.get_benchmark_shape_list import get_cnn_opset_shape_List
+from utils.helix_runtime import read_prof_dict
+from MI355X_FP32.MI355X_FP32_conv import get_MI355X_FP32_conv_Helix_result
+
+root_path = os.getcwd()
+
+
+def _summed_cost(prof_dict, shape_list, backend):
+    total = 0
+    for batch, input_channel, H, W, output_channel, kH, kW, stride, pad in shape_list:
+        if input_channel % 4 != 0:
+            continue   # first layers (IC=3) need the explicit im2col path, which this backend does not have yet
+        cost, _ = get_MI355X_FP32_conv_Helix_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, backend)
+        total += cost
+    return total
+
+
+def MI355X_FP32_Helix_model_level_CNN_benchmark(backend="hip"):
+    prof_dict = read_prof_dict("MI355X_FP32")
+
+    AlexNet_shape_list, ResNet_shape_list, GoogleNet_shape_list = get_cnn_opset_shape_List()
+
+    helix_AlexNet_cost = _summed_cost(prof_dict, AlexNet_shape_list, backend)
+    helix_ResNet_cost = _summed_cost(prof_dict, ResNet_shape_list, backend)
+    helix_GoogleNet_cost = _summed_cost(prof_dict, GoogleNet_shape_list, backend)
+
+    print(f'AlexNet: {helix_AlexNet_cost:.2f} ms, ResNet: {helix_ResNet_cost:.2f} ms, GoogleNet: {helix_GoogleNet_cost:.2f} ms')
+
+
+if __name__ == "__main__":
+
+    MI355X_FP32_Helix_model_level_CNN_benchmark(backend="hip")

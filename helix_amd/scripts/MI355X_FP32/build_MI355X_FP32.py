@@ -1,0 +1,117 @@
+"""Build step of the MI355X_FP32 backend: instantiate the FP32 MFMA SGEMM template space and compile
+every point with hipcc into its own shared library (plus the FP32 GEMV libraries).
+
+Mirrors scripts/Ampere_FP32/build_Ampere_FP32.py (is_valid_config :7-12, compile_sgemm :17-28, the six
+nested loops :43-50) with the same entry-point names modulo the backend tag.  The reference's
+register-tile parameters (TM, TN, WARP_ROW_THREAD, COPY_A/B) describe a CUDA-core thread tile; the
+MFMA template is parameterised by workgroup tile BM x BN, stage depth BK and wave tile WAVE_M x WAVE_N
+instead.  Unlike the reference, which fires `os.popen(nvcc ...)` without waiting (:28), the build
+returns only when every library exists, and it does build the FP32 GEMV (the reference never compiles
+gemv_template_fp32.cu, :59-61).
+"""
+import os
+from tqdm import tqdm
+
+from utils.helix_runtime import SRC_ROOT, bin_dir, compile_many
+
+root_path = os.getcwd()
+
+WAVE_TILE_LIST = [32, 64, 128]
+BLOCK_SCALE_LIST = [1, 2, 4]
+BK_LIST = [8, 16, 32]
+LDS_LIMIT = 160 * 1024
+
+
+def is_valid_config(BMt, BNt, BM, BN, BK=16, WAVE_M=64, WAVE_N=64):
+    # reference rules (build_Ampere_FP32.py:7-12): fewer than 512 threads' worth of tiles, tile extent bounds
+    if BMt * BNt * 64 > 512:
+        return False
+    if BM > 256 or BN > 256 or BM < 32 or BN < 32:
+        return False
+    # gfx950 resources
+    threads = 64 * BMt * BNt
+    if (BK * BM // 4) % threads or (BK * BN // 4) % threads:       # GEMM tile copy, 16-byte chunks along M / N
+        return False
+    if (BM * BK // 4) % threads or (BN * BK // 4) % threads:       # conv tile copy, 16-byte chunks along K
+        return False
+    if 2 * BK * (BM + 32 + BN + 32) * 4 > LDS_LIMIT:
+        return False
+    if WAVE_M * WAVE_N // 64 > 256:
+        return False
+    return True
+
+
+def iter_configs():
+    """Yields (BM, BN, BK, WAVE_M, WAVE_N) in build order."""
+    for WAVE_M in WAVE_TILE_LIST:
+        for WAVE_N in WAVE_TILE_LIST:
+            for BK in BK_LIST:
+                for BMt in BLOCK_SCALE_LIST:
+                    for BNt in BLOCK_SCALE_LIST:
+                        BM = BMt * WAVE_M
+                        BN = BNt * WAVE_N
+                        if not is_valid_config(BMt, BNt, BM, BN, BK, WAVE_M, WAVE_N):
+                            continue
+                        yield (BM, BN, BK, WAVE_M, WAVE_N)
+
+
+def sgemm_library(BM, BN, BK, WAVE_M, WAVE_N):
+    return f"{bin_dir('fp32')}/libsgemm_{BM}_{BN}_{BK}_{WAVE_M}_{WAVE_N}.so"
+
+
+def kernel_library(kernel_name):
+    return f"{bin_dir('fp32')}/lib{kernel_name}.so"
+
+
+def default_library():
+    """A mid-sized configuration used by smoke checks."""
+    return sgemm_library(128, 128, 16, 64, 64)
+
+
+def library_for_key(key):
+    """prof-dict key -> library.  key = (BM, BN, BK, WAVE_M, WAVE_N, LDS_STAGES, COPY_A, COPY_B) keeps the
+    reference's eight fields with BM, BN, BK in the same places (profile_Ampere_FP32.py:46); BK == 0 marks
+    the GEMV rows, whose first two fields are the activation-row tile and 128 weight rows."""
+    if key[2] == 0:
+        return kernel_library("gemv_fp32" if key[5] == 0 else "gemv_fp32_splitK")
+    return sgemm_library(key[0], key[1], key[2], key[3], key[4])
+
+
+def compile_sgemm(BM, BN, BK, WAVE_M, WAVE_N):
+    defines = {"BM": BM, "BN": BN, "BK": BK, "WAVE_M": WAVE_M, "WAVE_N": WAVE_N}
+    return (f"{SRC_ROOT}/MI355X_FP32/sgemm.hip", sgemm_library(BM, BN, BK, WAVE_M, WAVE_N), defines)
+
+
+def compile_kernel(kernel_name):
+    defines = {}
+    src_name = kernel_name
+    if kernel_name == "gemv_fp32_splitK":
+        src_name = "gemv_fp32"
+        defines["SPLIT_K"] = 4
+    return (f"{SRC_ROOT}/MI355X_FP32/{src_name}.hip", kernel_library(kernel_name), defines)
+
+
+def build_jobs():
+    jobs = [compile_sgemm(*cfg) for cfg in iter_configs()]
+    jobs.append(compile_kernel("gemv_fp32"))
+    jobs.append(compile_kernel("gemv_fp32_splitK"))
+    return jobs
+
+
+def build_Helix_MI355X_FP32_gemm_kernel():
+    if not os.path.exists(f"{root_path}/build/bin_fp32"):
+        os.makedirs(f"{root_path}/build/bin_fp32")
+
+    print("Start building MI355X FP32 GEMM kernel ...")
+    jobs = build_jobs()
+    with tqdm(total=len(jobs), desc="building") as pbar:
+        failed = compile_many(jobs, progress=pbar)
+    for out, err in failed:
+        print(f"Build failed: {out}\n{err}")
+    print("Build finished.")
+    return failed
+
+
+if __name__ == "__main__":
+
+    build_Helix_MI355X_FP32_gemm_kernel()

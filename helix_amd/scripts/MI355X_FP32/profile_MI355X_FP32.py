@@ -1,0 +1,66 @@
+"""Profile step of the MI355X_FP32 backend.  Mirrors scripts/Ampere_FP32/profile_Ampere_FP32.py:16-51
+(one timing per configuration, K = 1024, failures recorded as inf, dict literal on disk).  As in the FP16
+backend every configuration is timed on one full round of tiles over the 256 compute units rather than
+on one lonely tile."""
+import os
+from tqdm import tqdm
+
+from utils.helix_runtime import load, write_prof_dict
+from utils.roofline import NUM_CU
+from MI355X_FP32.build_MI355X_FP32 import iter_configs, library_for_key
+
+root_path = os.getcwd()
+
+PROFILE_K = 1024            # reference: K = 1024 (profile_Ampere_FP32.py:39)
+PROFILE_ROUNDS = 1
+PROFILE_GRID = 16
+GEMV_ROW_TILES = [1, 4, 16]
+GEMV_KEYS = [(mt, 128, 0, 0, 0, 0, 4, 4) for mt in GEMV_ROW_TILES]
+GEMV_SPLITK_KEYS = [(mt, 128, 0, 0, 0, 1, 4, 4) for mt in GEMV_ROW_TILES]
+GEMV_PROFILE_ROWS = 128 * NUM_CU
+GEMV_PROFILE_K = 4096
+
+
+def profile_problem(key):
+    if key[2] == 0:
+        return key[0], GEMV_PROFILE_ROWS, GEMV_PROFILE_K, 1
+    return key[0] * PROFILE_GRID, key[1] * PROFILE_GRID * PROFILE_ROUNDS, PROFILE_K, PROFILE_ROUNDS
+
+
+def time_config(key, warmup=3, iters=10):
+    M, N, K, rounds = profile_problem(key)
+    try:
+        lib = load(library_for_key(key))
+        rotate = (1 << 30) if key[2] == 0 else 0
+        _, avg, _ = lib.bench(M, N, K, warmup=warmup, iters=iters, outer=1, rotate_bytes=rotate)
+    except Exception as e:
+        print(f"Skip config {key}: {e}")
+        return float("inf")
+    return avg / rounds
+
+
+def all_keys():
+    keys = [(BM, BN, BK, WAVE_M, WAVE_N, 2, 4, 4) for (BM, BN, BK, WAVE_M, WAVE_N) in iter_configs()]
+    return keys + GEMV_KEYS + GEMV_SPLITK_KEYS
+
+
+def profile_Helix_MI355X_FP32_gemm_kernel():
+    if not os.path.exists(f"{root_path}/build/prof_dict"):
+        os.makedirs(f"{root_path}/build/prof_dict")
+
+    prof_dict = {}
+    print("Start profiling MI355X FP32 GEMM kernel ...")
+    keys = all_keys()
+    with tqdm(total=len(keys), desc="profiling") as pbar:
+        for key in keys:
+            prof_dict[key] = time_config(key)
+            pbar.update(1)
+
+    write_prof_dict("MI355X_FP32", prof_dict)
+    print("Profile finished.")
+    return prof_dict
+
+
+if __name__ == "__main__":
+
+    profile_Helix_MI355X_FP32_gemm_kernel()

@@ -1,0 +1,124 @@
+"""Shared host plumbing of the MI355X backends: hipcc invocation, artifact paths, library cache.
+
+The reference shells out once per configuration (`os.system("nvcc ... -o build/bin_fp16/gemm_...")`,
+scripts/Ampere_FP16/build_Ampere_FP16.py:7-28) and once per measurement (`os.popen(exe M N K)`,
+scripts/Ampere_FP16/profile_Ampere_FP16.py:36-38).  Here a configuration is a shared library that is
+compiled once, loaded once per process and called through ctypes.
+"""
+import os
+import subprocess
+import time
+from concurrent.futures import ThreadPoolExecutor
+
+from utils.hip_ctypes import HelixLib
+
+root_path = os.getcwd()
+
+_SCRIPTS_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC_ROOT = os.path.normpath(os.path.join(_SCRIPTS_DIR, "..", "src_template"))
+
+
+def _find_include_dir():
+    for cand in (os.path.join(_SCRIPTS_DIR, "..", "..", "include"), os.path.join(_SCRIPTS_DIR, "..", "include")):
+        if os.path.exists(os.path.join(cand, "helix_abi.h")):
+            return os.path.normpath(cand)
+    raise FileNotFoundError("include/helix_abi.h not found next to the scripts tree")
+
+
+HIPCC = os.environ.get("HIPCC", "hipcc")
+# -packed-fp32-ops is switched off on purpose: the compiler must not form packed FP32 VALU ops here.
+COMPILE_OPTIONS = ("-O3 -std=c++17 --offload-arch=gfx950 -shared -fPIC -w "
+                   "-Xclang -target-feature -Xclang -packed-fp32-ops")
+
+
+def bin_dir(precision):
+    return f"{root_path}/build/bin_{precision}"
+
+
+def prof_dict_path(backend):
+    return f"{root_path}/build/prof_dict/{backend}_cost_model.dict"
+
+
+def compile_command(src, out, defines):
+    inc = _find_include_dir()
+    cmd = f"{HIPCC} {src} {COMPILE_OPTIONS} -I{inc} -I{os.path.join(SRC_ROOT, 'common')}"
+    for k, v in defines.items():
+        cmd += f" -D{k}={v}"
+    cmd += f" -o {out}"
+    return cmd
+
+
+def compile_library(src, out, defines):
+    """Returns (ok, stderr_text)."""
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    tmp = out + ".tmp"
+    proc = subprocess.run(compile_command(src, tmp, defines), shell=True, capture_output=True, text=True)
+    if proc.returncode != 0:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+        return False, proc.stderr
+    os.replace(tmp, out)
+    return True, proc.stderr
+
+
+def compile_many(jobs, max_workers=None, progress=None):
+    """jobs: iterable of (src, out, defines).  Compiles in parallel; returns list of failed outs."""
+    jobs = list(jobs)
+    if max_workers is None:
+        max_workers = int(os.environ.get("MAX_JOBS", min(16, os.cpu_count() or 1)))
+    failed = []
+
+    def run(job):
+        ok, err = compile_library(*job)
+        return job, ok, err
+
+    with ThreadPoolExecutor(max_workers=max_workers) as ex:
+        for job, ok, err in ex.map(run, jobs):
+            if not ok:
+                failed.append((job[1], err))
+            if progress is not None:
+                progress.update(1)
+    return failed
+
+
+_lib_cache = {}
+
+
+def load(path):
+    """Process-wide cache of loaded kernel libraries (raises FileNotFoundError if not built)."""
+    lib = _lib_cache.get(path)
+    if lib is None:
+        lib = HelixLib(path)
+        _lib_cache[path] = lib
+    return lib
+
+
+def read_prof_dict(backend):
+    with open(prof_dict_path(backend), "r") as f:
+        lines = f.readlines()
+        # same `eval(lines[0])` as the reference (benchmark_Ampere_FP16_gemm.py:10-12); `inf` is bound because
+        # skipped configurations are stored as float('inf'), whose repr is not a Python literal
+        return eval(lines[0], {"inf": float("inf"), "nan": float("nan")})
+
+
+def write_prof_dict(backend, prof_dict):
+    os.makedirs(os.path.dirname(prof_dict_path(backend)), exist_ok=True)
+    with open(prof_dict_path(backend), "w") as f:
+        f.write(str(prof_dict))
+
+
+def reference_line(M, N, K, min_s, avg_s, max_s):
+    """The stdout line of the reference executables (src_template/Ampere_FP16/gemm.cu:687-689); its
+    whitespace-split token [-8] is the mean seconds, which is what the reference profilers parse."""
+    tflops = 2.0 * M * N * K / 1e12 / avg_s
+    return (f"M N K = {M:6d} {N:6d} {K:6d}, Time = {min_s:12.8f} {avg_s:12.8f} {max_s:12.8f} s, "
+            f"AVG Performance = {tflops:10.4f} Tflops")
+
+
+class Stopwatch:
+    def __enter__(self):
+        self.t0 = time.perf_counter()
+        return self
+
+    def __exit__(self, *a):
+        self.seconds = time.perf_counter() - self.t0

@@ -32,7 +32,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../../../include/helix_abi.h"
+#include "helix_abi.h"
 
 #ifndef BLOCK_ROWS
 #define BLOCK_ROWS 256
@@ -430,4 +430,4 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
 
 }  // namespace tpl
 
-#include "../common/helix_host.h"
+#include "helix_host.h"

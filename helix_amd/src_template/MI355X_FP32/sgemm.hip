@@ -1,0 +1,351 @@
+// MI355X (gfx950 / CDNA4) FP32 GEMM + implicit-GEMM convolution template on the FP32 matrix cores.
+//
+//   GEMM : C[M x N] = A^T * B with A stored K x M and B stored K x N (row-major FP32), the operand
+//          convention of the reference FP32 kernel (src_template/Ampere_FP32/sgemm.cu:138,378-382).
+//   CONV : y[B,OH,OW,OC] = conv2d(x[B,H,W,IC], w[OC,kH,kW,IC]), FP32, == GEMM with M = B*OH*OW, N = OC,
+//          K = kH*kW*IC; both operands are then K-contiguous and are transposed on their way into LDS.
+//
+// Role in the reference: src_template/Ampere_FP32/sgemm.cu:97-350 (`mySgemmCPAsyncTemplate`, a CUDA-core
+// register-tiled SGEMM with macros BM, BN, BK, TM, TN, :60-93).  Here the contraction runs on
+// v_mfma_f32_32x32x2_f32: one wave64 owns a WAVE_M x WAVE_N tile made of 32x32 MFMA tiles, each MFMA
+// consuming two k values; products are accumulated in ascending k, the same order the CPU path uses.
+//
+// Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N.
+//
+// LDS layout: A stage is [BK][BM + 32] floats, B stage [BK][BN + 32]; a fragment read takes lanes 0-31
+// from row k and lanes 32-63 from row k+1, and the 32-float row padding puts the two half-waves on
+// different halves of the 64 banks.  In CONV mode operands arrive K-contiguous and are written
+// transposed into the same layout.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "helix_abi.h"
+
+#ifndef BM
+#define BM 128
+#endif
+#ifndef BN
+#define BN 128
+#endif
+#ifndef BK
+#define BK 16
+#endif
+#ifndef WAVE_M
+#define WAVE_M 64
+#endif
+#ifndef WAVE_N
+#define WAVE_N 64
+#endif
+#ifndef GROUP_ROWS
+#define GROUP_ROWS 8
+#endif
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef int intx4 __attribute__((ext_vector_type(4)));
+
+constexpr int WAVES_M = BM / WAVE_M, WAVES_N = BN / WAVE_N, NWAVES = WAVES_M * WAVES_N, NTHREADS = 64 * NWAVES;
+constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;
+constexpr int LDA_S = BM + 32, LDB_S = BN + 32;              // LDS row strides in floats
+constexpr int A_STAGE = BK * LDA_S, B_STAGE = BK * LDB_S;    // floats
+constexpr int STAGE = A_STAGE + B_STAGE;
+constexpr int LDS_BYTES = 2 * STAGE * 4;
+// GEMM mode: tile rows are k, 16-byte chunks run along m / n
+constexpr int A_CPR = BM / 4, B_CPR = BN / 4;                // chunks per tile row
+constexpr int A_ITERS = BK * A_CPR / NTHREADS, B_ITERS = BK * B_CPR / NTHREADS;
+// CONV mode: tile rows are m / n, 16-byte chunks run along k
+constexpr int K_CPR = BK / 4;
+constexpr int AC_ITERS = BM * K_CPR / NTHREADS, BC_ITERS = BN * K_CPR / NTHREADS;
+
+static_assert(BM % WAVE_M == 0 && BN % WAVE_N == 0, "block tile must be a multiple of the wave tile");
+static_assert(WAVE_M % 32 == 0 && WAVE_N % 32 == 0, "wave tile is built from 32x32 MFMA tiles");
+static_assert(BK % 4 == 0 && BK >= 4, "BK must be a multiple of 4");
+static_assert(NTHREADS <= 1024, "too many waves");
+static_assert((BK * A_CPR) % NTHREADS == 0 && (BK * B_CPR) % NTHREADS == 0, "tile copy must divide evenly");
+static_assert((BM * K_CPR) % NTHREADS == 0 && (BN * K_CPR) % NTHREADS == 0, "conv tile copy must divide evenly");
+static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
+
+struct ConvGeom {
+    int H, W, IC, OH, OW, kW, stride, pad, M;
+};
+
+struct Params {
+    const float* A;  // GEMM: K x M (lda).  CONV: x, NHWC
+    const float* B;  // GEMM: K x N (ldb).  CONV: w, [OC][kH][kW][IC]
+    float* C;        // M x N (ldc)
+    int M, N, K, lda, ldb, ldc;
+    int tiles_m, tiles_n;
+    unsigned a_bytes;
+    ConvGeom g;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ floatx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) {
+    return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+}
+
+constexpr int OOB = 0x7fffffff;  // byte offset beyond any buffer: the load returns zeros
+
+template <bool CONV>
+__global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params p) {
+    extern __shared__ __attribute__((aligned(16))) float smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+
+    // workgroup id -> tile: undo the round-robin deal over the 8 XCDs, then walk groups of tile rows
+    const int ntiles = p.tiles_m * p.tiles_n;
+    int pid = blockIdx.x;
+    {
+        const int per = ntiles / 8, rem = ntiles % 8;
+        const int xcd = pid % 8, slot = pid / 8;
+        pid = xcd * per + (xcd < rem ? xcd : rem) + slot;
+    }
+    const int group_tiles = GROUP_ROWS * p.tiles_n;
+    const int first_m = (pid / group_tiles) * GROUP_ROWS;
+    const int gsize = (p.tiles_m - first_m) < GROUP_ROWS ? (p.tiles_m - first_m) : GROUP_ROWS;
+    const int tile_m = first_m + (pid % group_tiles) % gsize;
+    const int tile_n = (pid % group_tiles) / gsize;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    constexpr int NA = CONV ? AC_ITERS : A_ITERS;
+    constexpr int NB = CONV ? BC_ITERS : B_ITERS;
+    floatx4 stage_a[NA], stage_b[NB];
+
+    // CONV: per-row gather state
+    int cv_img[NA], cv_ih[NA], cv_iw[NA];
+    if (CONV) {
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            const int m = m0 + (tid + i * NTHREADS) / K_CPR;
+            const int ow = m % p.g.OW;
+            const int t = m / p.g.OW;
+            const int oh = t % p.g.OH;
+            const int b = t / p.g.OH;
+            cv_img[i] = (m < p.g.M) ? b * p.g.H * p.g.W : -1;
+            cv_ih[i] = oh * p.g.stride - p.g.pad;
+            cv_iw[i] = ow * p.g.stride - p.g.pad;
+        }
+    }
+
+    auto load_global = [&](int k0) {
+        if (!CONV) {
+            // rows k0.. of A^T (K x M) starting at column m0; whole rows are inside the buffer, rows >= K are not
+            __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + (size_t)k0 * p.lda + m0,
+                                                  (unsigned)(((size_t)(p.K - k0) * p.lda - m0) * 4));
+            __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)k0 * p.ldb + n0,
+                                                  (unsigned)(((size_t)(p.K - k0) * p.ldb - n0) * 4));
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                const int c = tid + i * NTHREADS;
+                stage_a[i] = buf_load16(ra, ((c / A_CPR) * p.lda + (c % A_CPR) * 4) * 4);
+            }
+#pragma unroll
+            for (int i = 0; i < NB; i++) {
+                const int c = tid + i * NTHREADS;
+                stage_b[i] = buf_load16(rb, ((c / B_CPR) * p.ldb + (c % B_CPR) * 4) * 4);
+            }
+        } else {
+            __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, p.a_bytes);
+            const int kc = tid % K_CPR;
+            const int k = k0 + kc * 4;
+            const bool dead = k >= p.K;
+            const int c = k % p.g.IC;
+            const int t = k / p.g.IC;
+            const int kw = t % p.g.kW;
+            const int kh = t / p.g.kW;
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
+                const bool ok = !dead && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W;
+                stage_a[i] = buf_load16(ra, ok ? ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 4 : OOB);
+            }
+            // weights: N x K row-major; rows >= N fall outside the buffer
+            const int rows_b = (p.N - n0) < BN ? (p.N - n0) : BN;
+            __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)n0 * p.K, (unsigned)((size_t)rows_b * p.K * 4));
+#pragma unroll
+            for (int i = 0; i < NB; i++) {
+                const int n = (tid + i * NTHREADS) / K_CPR;
+                stage_b[i] = buf_load16(rb, dead ? OOB : (n * p.K + k) * 4);
+            }
+        }
+    };
+
+    auto store_lds = [&](int stage) {
+        float* sa = smem + stage * STAGE;
+        float* sb = sa + A_STAGE;
+        if (!CONV) {
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                const int c = tid + i * NTHREADS;
+                *(floatx4*)(sa + (c / A_CPR) * LDA_S + (c % A_CPR) * 4) = stage_a[i];
+            }
+#pragma unroll
+            for (int i = 0; i < NB; i++) {
+                const int c = tid + i * NTHREADS;
+                *(floatx4*)(sb + (c / B_CPR) * LDB_S + (c % B_CPR) * 4) = stage_b[i];
+            }
+        } else {
+            const int kc = (tid % K_CPR) * 4;
+#pragma unroll
+            for (int i = 0; i < NA; i++) {
+                const int m = (tid + i * NTHREADS) / K_CPR;
+#pragma unroll
+                for (int e = 0; e < 4; e++) sa[(kc + e) * LDA_S + m] = stage_a[i][e];
+            }
+#pragma unroll
+            for (int i = 0; i < NB; i++) {
+                const int n = (tid + i * NTHREADS) / K_CPR;
+#pragma unroll
+                for (int e = 0; e < 4; e++) sb[(kc + e) * LDB_S + n] = stage_b[i][e];
+            }
+        }
+    };
+
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+
+    // MFMA 32x32x2: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32]
+    const int frow = lane & 31, fk = lane >> 5;
+    const int a_rd = fk * LDA_S + wave_m * WAVE_M + frow;
+    const int b_rd = A_STAGE + fk * LDB_S + wave_n * WAVE_N + frow;
+
+    const int ktiles = (p.K + BK - 1) / BK;
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < ktiles; kt++) {
+        const int cur = kt & 1;
+        const bool more = (kt + 1 < ktiles);
+        if (more) load_global((kt + 1) * BK);
+
+        const float* sb = smem + cur * STAGE;
+#pragma unroll
+        for (int s = 0; s < BK / 2; s++) {
+            float af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) af[i] = sb[a_rd + s * 2 * LDA_S + i * 32];
+#pragma unroll
+            for (int j = 0; j < TN; j++) bf[j] = sb[b_rd + s * 2 * LDB_S + j * 32];
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+
+        if (more) store_lds(cur ^ 1);
+        __syncthreads();
+    }
+
+    // lane l holds column (l % 32); rows 8*(v/4) + 4*(l/32) + (v%4)
+    const int col_l = lane & 31, row_l = (lane >> 5) * 4;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = n0 + wave_n * WAVE_N + j * 32 + col_l;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int row = m0 + wave_m * WAVE_M + i * 32 + (v / 4) * 8 + row_l + (v % 4);
+                if (row < p.M && col < p.N) p.C[(size_t)row * p.ldc + col] = acc[i][j][v];
+            }
+        }
+    }
+}
+
+}  // namespace
+
+#include <stdio.h>
+
+namespace tpl {
+
+constexpr int kElemBytes = 4;
+
+inline const char* info_json() {
+    static char buf[1024];
+    static bool done = false;
+    if (!done) {
+        snprintf(buf, sizeof(buf),
+                 "{\"family\": \"sgemm_f32\", \"arch\": \"gfx950\", \"mfma\": \"v_mfma_f32_32x32x2_f32\", "
+                 "\"lds_stages\": 2, \"block_rows\": %d, \"block_cols\": %d, \"wave_rows\": %d, \"wave_cols\": %d, "
+                 "\"block_k\": %d, \"split_k\": 1, \"threads\": %d, \"lds_bytes\": %d, "
+                 "\"layout_a\": \"K x M row-major f32 (A transposed)\", \"layout_b\": \"K x N row-major f32\", "
+                 "\"layout_c\": \"M x N row-major f32\", \"accumulate\": \"f32\", "
+                 "\"k_multiple\": 1, \"ld_multiple\": 4, \"conv\": \"NHWC x [OC][kH][kW][IC], IC %% 4 == 0\"}",
+                 BM, BN, WAVE_M, WAVE_N, BK, NTHREADS, LDS_BYTES);
+        done = true;
+    }
+    return buf;
+}
+
+inline size_t workspace_bytes(int, int, int) { return 0; }
+
+inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce, int* lda, int* ldb, int* ldc) {
+    const int Mp = (M + 3) / 4 * 4, Np = (N + 3) / 4 * 4;
+    *ae = (size_t)K * Mp; *be = (size_t)K * Np; *ce = (size_t)M * Np;
+    *lda = Mp; *ldb = Np; *ldc = Np;
+}
+
+template <bool CONV>
+inline int launch(const Params& p, hipStream_t s) {
+    static int rc = (int)hipFuncSetAttribute((const void*)helix_sgemm_f32_kernel<CONV>,
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
+    if (rc) return rc;
+    const long long ntiles = (long long)p.tiles_m * p.tiles_n;
+    if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    hipLaunchKernelGGL(helix_sgemm_f32_kernel<CONV>, dim3((unsigned)ntiles), dim3(NTHREADS), LDS_BYTES, s, p);
+    return (int)hipGetLastError();
+}
+
+inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc, void*, size_t,
+                hipStream_t s) {
+    if (lda % 4 != 0 || ldb % 4 != 0) return HELIX_ERR_INVALID_VALUE;  // 16-byte loads along M and N
+    if (lda < M || ldb < N || ldc < N) return HELIX_ERR_INVALID_VALUE;
+    if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)C & 3)) return HELIX_ERR_INVALID_VALUE;
+    // byte offsets inside one K tile are 32-bit, and a buffer descriptor spans at most 4 GiB
+    if ((long long)K * lda * 4 >= 0xffffffffLL || (long long)K * ldb * 4 >= 0xffffffffLL)
+        return HELIX_ERR_INVALID_VALUE;
+    if ((long long)BK * lda * 4 >= 0x7fffffffLL || (long long)BK * ldb * 4 >= 0x7fffffffLL)
+        return HELIX_ERR_INVALID_VALUE;
+    Params p{};
+    p.A = (const float*)A; p.B = (const float*)B; p.C = (float*)C;
+    p.M = M; p.N = N; p.K = K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+    p.tiles_m = (M + BM - 1) / BM; p.tiles_n = (N + BN - 1) / BN;
+    return launch<false>(p, s);
+}
+
+inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
+                  int stride, int pad, void*, size_t, hipStream_t s) {
+    if (IC % 4 != 0) return HELIX_ERR_INVALID_VALUE;  // a 16-byte chunk must stay inside one filter tap
+    const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
+    const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
+    const long long xbytes = (long long)batch * H * W * IC * 4;
+    if (M > 0x7fffffffLL || K > 0x7fffffffLL || xbytes >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    if ((long long)BN * K * 4 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 3)) return HELIX_ERR_INVALID_VALUE;
+    Params p{};
+    p.A = (const float*)x; p.B = (const float*)w; p.C = (float*)y;
+    p.M = (int)M; p.N = OC; p.K = (int)K; p.lda = 0; p.ldb = (int)K; p.ldc = OC;
+    p.tiles_m = (int)((M + BM - 1) / BM); p.tiles_n = (OC + BN - 1) / BN;
+    p.a_bytes = (unsigned)xbytes;
+    p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M};
+    return launch<true>(p, s);
+}
+
+}  // namespace tpl
+
+#include "helix_host.h"

@@ -26,7 +26,7 @@
 #include <float.h>
 #include <vector>
 
-#include "../../../include/helix_abi.h"
+#include "helix_abi.h"
 
 #define HELIX_HIP_TRY(expr)                      \
     do {                                         \

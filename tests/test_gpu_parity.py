@@ -1,0 +1,444 @@
+"""GPU parity tests: every kernel family is called through the C ABI (ctypes -> helix_gemm / helix_conv2d)
+and compared with the CPU oracle on the same seeded inputs.
+
+Tolerances (normwise: |got - want| <= tol * max|want|, because the inputs are zero-mean and an elementwise
+relative error is unbounded near zero):
+    FP16 in / FP32 accumulate / FP16 out : 2e-2   (the stated bound; observed values are ~5e-4)
+    FP32                                 : 1e-5
+Integer-valued inputs make FP32 accumulation exact, so tile / edge / split-K mistakes show as exact
+mismatches in those cases.
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from utils import seeded_inputs
+from utils.helix_runtime import load
+from utils.hip_ctypes import HelixError, HELIX_ERR_INVALID_VALUE, HELIX_ERR_UNSUPPORTED, HELIX_ERR_WORKSPACE
+from MI355X_FP16 import build_MI355X_FP16 as b16
+from MI355X_FP32 import build_MI355X_FP32 as b32
+
+pytestmark = pytest.mark.gpu
+
+TOL16 = 2e-2
+TOL32 = 1e-5
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
+
+
+def normwise(got, want):
+    want = np.asarray(want, dtype=np.float64)
+    return float(np.max(np.abs(np.asarray(got, dtype=np.float64) - want)) / max(np.max(np.abs(want)), 1e-30))
+
+
+def run_gemm_f16(lib, A, B, ldpad=0):
+    """A (M,K) f16, B (K,N) f16 -> C (M,N) f16 through helix_gemm (device layout: B as N x K)."""
+    M, K = A.shape
+    N = B.shape[1]
+    Kp = (K + 7) // 8 * 8 + ldpad
+    Ap = np.zeros((M, Kp), np.float16)
+    Ap[:, :K] = A
+    Bt = np.zeros((N, Kp), np.float16)
+    Bt[:, :K] = B.T
+    dA, dB = dev(Ap), dev(Bt)
+    dC = torch.full((M, N), float("nan"), dtype=torch.float16, device="cuda:0")
+    Kk = (K + 7) // 8 * 8
+    wsb = lib.workspace_bytes(M, N, Kk)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda:0")
+    lib.gemm(dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), M, N, Kk, Kp, Kp, N, ws.data_ptr(), wsb,
+             torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return dC.cpu().numpy()
+
+
+def run_sgemm_f32(lib, A, B):
+    """A (M,K) f32, B (K,N) f32 -> C (M,N) f32 through helix_gemm (device layout: A as K x M)."""
+    M, K = A.shape
+    N = B.shape[1]
+    Mp, Np = (M + 3) // 4 * 4, (N + 3) // 4 * 4
+    At = np.zeros((K, Mp), np.float32)
+    At[:, :M] = A.T
+    Bp = np.zeros((K, Np), np.float32)
+    Bp[:, :N] = B
+    dA, dB = dev(At), dev(Bp)
+    dC = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda:0")
+    lib.gemm(dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), M, N, K, Mp, Np, N, 0, 0,
+             torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return dC.cpu().numpy()
+
+
+FP16_CONFIGS = [(2, 256, 256, 128, 128, 64), (2, 256, 256, 64, 128, 64), (2, 128, 128, 64, 64, 32), (2, 64, 64, 32, 32, 64),
+                (2, 32, 32, 32, 32, 32), (2, 256, 64, 64, 32, 64), (2, 64, 256, 32, 128, 32), (2, 128, 256, 128, 64, 64)]
+
+
+# ---------------------------------------------------------------------------------------------
+# FP16 GEMM
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("cfg", FP16_CONFIGS)
+@pytest.mark.parametrize("splitk", [0, 1])
+def test_gemm_f16_vs_oracle(cfg, splitk):
+    lib = load(b16.kernel_library("gemm_splitK" if splitk else "gemm", *cfg))
+    for (M, N, K) in [(256, 256, 256), (300, 200, 136), (1, 7, 8), (513, 1025, 72), (1024, 1024, 1024)]:
+        A, B = seeded_inputs.gemm_operands(M, N, K, np.float16)
+        got = run_gemm_f16(lib, A, B)
+        want = O.hgemm_f32acc(A, B)
+        assert not np.isnan(got).any(), (cfg, M, N, K)
+        assert normwise(got, want) < TOL16, (cfg, M, N, K)
+
+
+@pytest.mark.parametrize("cfg", FP16_CONFIGS[:4])
+def test_gemm_f16_integer_inputs_exact(cfg):
+    """Small integers: products and FP32 sums are exact, and the sums are kept below 2048 in magnitude so
+    the FP16 result is exact too -- any wrong tile, edge or split-K index is an exact mismatch."""
+    rng = np.random.default_rng(3)
+    for splitk in (0, 1):
+        lib = load(b16.kernel_library("gemm_splitK" if splitk else "gemm", *cfg))
+        for (M, N, K) in [(257, 129, 200), (64, 500, 328)]:
+            A = rng.integers(-2, 3, (M, K)).astype(np.float16)
+            B = rng.integers(-2, 3, (K, N)).astype(np.float16)
+            want = A.astype(np.int64) @ B.astype(np.int64)
+            assert np.abs(want).max() < 2048
+            got = run_gemm_f16(lib, A, B)
+            assert np.array_equal(got.astype(np.int64), want), (cfg, splitk, M, N, K)
+            assert np.array_equal(O.hgemm_f32acc(A, B).astype(np.int64), want)
+
+
+def test_gemm_f16_closed_forms_and_layout():
+    lib = load(b16.kernel_library("gemm", 2, 128, 128, 64, 64, 64))
+    rng = np.random.default_rng(4)
+    B = (rng.standard_normal((160, 96)) * 0.5).astype(np.float16)
+    # identity picks B exactly; a unit vector e_i e_j^T moves row j of B to row i (transposed operands fail this)
+    assert np.array_equal(run_gemm_f16(lib, np.eye(160, dtype=np.float16), B), B)
+    E = np.zeros((40, 160), np.float16)
+    E[7, 150] = 1
+    want = np.zeros((40, 96), np.float16)
+    want[7] = B[150]
+    assert np.array_equal(run_gemm_f16(lib, E, B), want)
+    # ones: C == K, exact up to 2048
+    assert np.array_equal(run_gemm_f16(lib, np.ones((33, 2048), np.float16), np.ones((2048, 65), np.float16)),
+                          np.full((33, 65), 2048, np.float16))
+    # row strides larger than K (padded leading dimensions) do not leak into the result
+    A = (rng.standard_normal((100, 160)) * 0.1).astype(np.float16)
+    assert normwise(run_gemm_f16(lib, A, B, ldpad=24), O.hgemm_f32acc(A, B)) < TOL16
+
+
+def test_gemm_f16_golden_vectors():
+    lib = load(b16.kernel_library("gemm", 2, 64, 64, 32, 32, 32))
+    files = sorted(glob.glob(os.path.join(GOLDEN, "gemm_f16_*.npz")))
+    assert files
+    for f in files:
+        d = np.load(f)
+        got = run_gemm_f16(lib, d["A"], d["B"])
+        assert normwise(got, d["C64"]) < TOL16, f
+        assert normwise(got, O.hgemm_f32acc(d["A"], d["B"])) < TOL16, f
+
+
+def test_gemm_f16_full_size_properties():
+    """8192^3 (the benchmark size): too big for the CPU oracle in seconds, so check size-independent facts:
+    a random sample of outputs against float64 dot products, and linearity in A."""
+    M = N = K = 8192
+    lib = load(b16.kernel_library("gemm", 2, 256, 256, 128, 128, 64))
+    A, B = seeded_inputs.gemm_operands(M, N, K, np.float16)
+    Bt = np.ascontiguousarray(B.T)
+    dA, dB = dev(A), dev(Bt)
+    dC = torch.empty((M, N), dtype=torch.float16, device="cuda:0")
+    lib.gemm(dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), M, N, K, K, K, N)
+    torch.cuda.synchronize()
+    C = dC.cpu().numpy()
+    rng = np.random.default_rng(5)
+    rows, cols = rng.integers(0, M, 256), rng.integers(0, N, 256)
+    want = np.einsum("ik,ik->i", A[rows].astype(np.float64), Bt[cols].astype(np.float64))
+    scale = np.abs(want).max()
+    assert np.max(np.abs(C[rows, cols].astype(np.float64) - want)) < TOL16 * scale
+    # corners and tile seams
+    for (r, c) in [(0, 0), (M - 1, N - 1), (255, 256), (256, 255), (4095, 4096), (8191, 0)]:
+        w = float(A[r].astype(np.float64) @ Bt[c].astype(np.float64))
+        assert abs(float(C[r, c]) - w) < TOL16 * scale
+    # linearity: (2A) B == 2 (A B) exactly -- scaling by 2 is exact in FP16 and FP32 -- wherever the FP16
+    # result is a normal number (a subnormal result rounds on a fixed grid, where round(2x) != 2 round(x))
+    dA2 = dA * 2
+    dC2 = torch.empty_like(dC)
+    lib.gemm(dA2.data_ptr(), dB.data_ptr(), dC2.data_ptr(), M, N, K, K, K, N)
+    torch.cuda.synchronize()
+    normal = dC.abs() >= 2.0 ** -13
+    assert normal.float().mean().item() > 0.999
+    assert torch.equal(dC2[normal], (dC * 2)[normal])
+    assert (dC2.float() - 2 * dC.float()).abs().max().item() <= 2.0 ** -23
+
+
+def test_gemm_f16_rejects_bad_arguments():
+    lib = load(b16.kernel_library("gemm", 2, 128, 128, 64, 64, 64))
+    A = torch.zeros((64, 64), dtype=torch.float16, device="cuda:0")
+    C = torch.zeros((64, 64), dtype=torch.float16, device="cuda:0")
+    p = A.data_ptr()
+    assert lib.gemm(p, p, C.data_ptr(), 64, 64, 60, 64, 64, 64, check=False) == HELIX_ERR_INVALID_VALUE   # K % 8
+    assert lib.gemm(p, p, C.data_ptr(), 64, 64, 64, 60, 64, 64, check=False) == HELIX_ERR_INVALID_VALUE   # lda % 8
+    assert lib.gemm(p, p, C.data_ptr(), 64, 64, 64, 32, 64, 64, check=False) == HELIX_ERR_INVALID_VALUE   # lda < K
+    assert lib.gemm(p + 2, p, C.data_ptr(), 32, 32, 32, 64, 64, 64, check=False) == HELIX_ERR_INVALID_VALUE  # alignment
+    assert lib.gemm(0, p, C.data_ptr(), 64, 64, 64, 64, 64, 64, check=False) == HELIX_ERR_INVALID_VALUE
+    assert lib.gemm(p, p, C.data_ptr(), 0, 64, 64, 64, 64, 64, check=False) == HELIX_ERR_INVALID_VALUE
+    with pytest.raises(HelixError):
+        lib.gemm(p, p, C.data_ptr(), 64, 64, 60, 64, 64, 64)
+    sk = load(b16.kernel_library("gemm_splitK", 2, 128, 128, 64, 64, 64))
+    assert sk.workspace_bytes(64, 64, 64) == 2 * 64 * 64 * 4
+    assert sk.gemm(p, p, C.data_ptr(), 64, 64, 64, 64, 64, 64, 0, 0, check=False) == HELIX_ERR_WORKSPACE
+
+
+# ---------------------------------------------------------------------------------------------
+# FP16 GEMV
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["gemv", "gemv_splitK"])
+def test_gemv_f16_vs_oracle(name):
+    lib = load(b16.kernel_library(name))
+    for M in (1, 2, 3, 4, 5, 8, 16, 17):
+        for (N, K) in [(128, 512), (1000, 1032), (4096, 4096), (9001, 520), (20000, 8)]:
+            x, W = seeded_inputs.gemv_operands(M, N, K)
+            got = run_gemm_f16(lib, x, W)
+            want = O.hgemm_f32acc(x, W)
+            assert not np.isnan(got).any(), (M, N, K)
+            assert normwise(got, want) < TOL16, (M, N, K)
+
+
+def test_gemv_f16_integer_inputs_exact():
+    rng = np.random.default_rng(6)
+    for name in ("gemv", "gemv_splitK"):
+        lib = load(b16.kernel_library(name))
+        for (M, N, K) in [(1, 777, 1536), (4, 2050, 520), (16, 300, 1024), (7, 4100, 2056)]:
+            x = rng.integers(-2, 3, (M, K)).astype(np.float16)
+            W = rng.integers(-1, 2, (K, N)).astype(np.float16)
+            want = x.astype(np.int64) @ W.astype(np.int64)
+            assert np.abs(want).max() < 2048
+            assert np.array_equal(run_gemm_f16(lib, x, W).astype(np.int64), want), (name, M, N, K)
+
+
+def test_gemv_f16_baseline_shapes_sampled():
+    """The decode shapes at full size: sampled outputs against float64 dot products."""
+    lib = load(b16.kernel_library("gemv"))
+    rng = np.random.default_rng(7)
+    for (K, N) in [(4096, 11008), (8192, 28672)]:
+        for M in (1, 16):
+            x, W = seeded_inputs.gemv_operands(M, N, K)
+            Wt = np.ascontiguousarray(W.T)
+            dx, dW = dev(x), dev(Wt)
+            dy = torch.empty((M, N), dtype=torch.float16, device="cuda:0")
+            lib.gemm(dx.data_ptr(), dW.data_ptr(), dy.data_ptr(), M, N, K, K, K, N)
+            torch.cuda.synchronize()
+            y = dy.cpu().numpy()
+            cols = np.concatenate([rng.integers(0, N, 200), [0, N - 1]])
+            want = x.astype(np.float64) @ Wt[cols].astype(np.float64).T
+            assert np.max(np.abs(y[:, cols] - want)) < TOL16 * np.abs(want).max()
+
+
+def test_gemv_has_no_conv_entry():
+    lib = load(b16.kernel_library("gemv"))
+    t = torch.zeros(4096, dtype=torch.float16, device="cuda:0")
+    assert lib.conv2d(t.data_ptr(), t.data_ptr(), t.data_ptr(), 1, 4, 4, 8, 8, 1, 1, 1, 0, check=False) == \
+        HELIX_ERR_UNSUPPORTED
+
+
+# ---------------------------------------------------------------------------------------------
+# FP16 implicit-GEMM convolution
+# ---------------------------------------------------------------------------------------------
+def run_conv(lib, x, w, stride, pad, dtype):
+    batch, H, W, IC = x.shape
+    OC, kH, kW, _ = w.shape
+    OH, OW = O.conv_out_hw(H, W, kH, kW, stride, pad)
+    dx, dw = dev(x), dev(w)
+    dy = torch.full((batch, OH, OW, OC), float("nan"), dtype=dtype, device="cuda:0")
+    lib.conv2d(dx.data_ptr(), dw.data_ptr(), dy.data_ptr(), batch, H, W, IC, OC, kH, kW, stride, pad, 0, 0,
+               torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return dy.cpu().numpy()
+
+
+CONV_GEOMS = [(2, 14, 14, 16, 24, 3, 3, 1, 1), (2, 15, 13, 8, 8, 3, 3, 2, 1), (3, 8, 8, 32, 16, 1, 1, 2, 0),
+              (1, 12, 12, 8, 40, 5, 5, 1, 2), (2, 9, 9, 64, 64, 3, 3, 1, 1), (1, 7, 7, 24, 16, 3, 3, 1, 0),
+              (2, 6, 10, 72, 8, 1, 1, 1, 0)]
+
+
+@pytest.mark.parametrize("cfg", [(2, 128, 128, 64, 64, 64), (2, 64, 64, 32, 32, 32), (2, 256, 64, 64, 32, 64),
+                                 (2, 128, 64, 64, 32, 32)])
+def test_conv_f16_vs_oracle(cfg):
+    lib = load(b16.kernel_library("gemm", *cfg))
+    for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS:
+        x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW)
+        got = run_conv(lib, x, w, stride, pad, torch.float16)
+        want = O.conv2d_nhwc(x, w, stride, pad)
+        assert got.shape == want.shape
+        assert not np.isnan(got).any(), (cfg, batch, H, W, IC, OC, kH, kW, stride, pad)
+        assert normwise(got, want) < TOL16, (cfg, batch, H, W, IC, OC, kH, kW, stride, pad)
+
+
+def test_conv_f16_golden_and_special_cases():
+    lib = load(b16.kernel_library("gemm", 2, 64, 64, 32, 32, 32))
+    for f in sorted(glob.glob(os.path.join(GOLDEN, "conv_f16_*.npz"))):
+        d = np.load(f)
+        got = run_conv(lib, d["x"], d["w"], int(d["stride"]), int(d["pad"]), torch.float16)
+        assert normwise(got, d["y64"]) < TOL16, f
+    # 1x1 stride 1 == GEMM on the reshaped tensors: bit-identical to the GEMM entry point of the same library
+    x, w = seeded_inputs.conv_operands(2, 64, 12, 12, 48, 1, 1)
+    y = run_conv(lib, x, w, 1, 0, torch.float16)
+    g = run_gemm_f16(lib, x.reshape(-1, 64), np.ascontiguousarray(w.reshape(48, 64).T))
+    assert np.array_equal(y.reshape(-1, 48), g)
+    # integer-valued inputs: exact, padding taps contribute exactly zero
+    rng = np.random.default_rng(8)
+    xi = rng.integers(-2, 3, (2, 9, 8, 8)).astype(np.float16)
+    wi = rng.integers(-2, 3, (16, 3, 3, 8)).astype(np.float16)
+    want = O.conv2d_nhwc(xi.astype(np.float32), wi.astype(np.float32), 2, 1)
+    assert np.array_equal(run_conv(lib, xi, wi, 2, 1, torch.float16).astype(np.float32), want)
+    # unsupported channel count is refused, not mis-computed
+    t = torch.zeros(4096, dtype=torch.float16, device="cuda:0")
+    assert lib.conv2d(t.data_ptr(), t.data_ptr(), t.data_ptr(), 1, 8, 8, 3, 8, 3, 3, 1, 1, check=False) == \
+        HELIX_ERR_INVALID_VALUE
+
+
+def test_conv_f16_baseline_layers_sampled():
+    """The six ResNet-50-shaped layers at batch 32: sampled output pixels against float64."""
+    from utils.get_benchmark_shape_list import get_baseline_conv_shape_list
+    lib = load(b16.kernel_library("gemm", 2, 128, 64, 64, 32, 64))
+    rng = np.random.default_rng(9)
+    for (batch, IC, H, W, OC, kH, kW, stride, pad) in get_baseline_conv_shape_list():
+        x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW)
+        y = run_conv(lib, x, w, stride, pad, torch.float16)
+        OH, OW = O.conv_out_hw(H, W, kH, kW, stride, pad)
+        assert y.shape == (batch, OH, OW, OC)
+        xp = np.zeros((batch, H + 2 * pad, W + 2 * pad, IC), np.float64)
+        xp[:, pad:pad + H, pad:pad + W] = x
+        w64 = w.astype(np.float64)
+        pts = [(0, 0, 0), (batch - 1, OH - 1, OW - 1), (batch - 1, 0, OW - 1)] + \
+              [(int(rng.integers(batch)), int(rng.integers(OH)), int(rng.integers(OW))) for _ in range(40)]
+        worst, scale = 0.0, 0.0
+        for (b, oh, ow) in pts:
+            patch = xp[b, oh * stride:oh * stride + kH, ow * stride:ow * stride + kW]
+            want = np.einsum("hwc,ohwc->o", patch, w64)
+            worst = max(worst, np.max(np.abs(y[b, oh, ow] - want)))
+            scale = max(scale, np.max(np.abs(want)))
+        assert worst < TOL16 * scale, (batch, IC, H, W, OC, kH, kW, stride, pad)
+
+
+# ---------------------------------------------------------------------------------------------
+# FP32
+# ---------------------------------------------------------------------------------------------
+FP32_CONFIGS = [(128, 128, 16, 64, 64), (256, 128, 16, 128, 64), (32, 32, 8, 32, 32), (64, 256, 32, 32, 128),
+                (128, 64, 32, 64, 32)]
+
+
+@pytest.mark.parametrize("cfg", FP32_CONFIGS)
+def test_sgemm_f32_vs_oracle(cfg):
+    lib = load(b32.sgemm_library(*cfg))
+    for (M, N, K) in [(256, 256, 256), (300, 200, 137), (1, 7, 3), (513, 1025, 70), (1024, 1024, 1024)]:
+        A = seeded_inputs.uniform_pm1((M, K), seeded_inputs.SEED_A)
+        B = seeded_inputs.uniform_pm1((K, N), seeded_inputs.SEED_B)
+        got = run_sgemm_f32(lib, A, B)
+        want = O.sgemm_seqk(A, B)
+        assert not np.isnan(got).any(), (cfg, M, N, K)
+        assert normwise(got, want) < TOL32, (cfg, M, N, K)
+
+
+def test_sgemm_f32_exact_and_closed_forms():
+    lib = load(b32.sgemm_library(128, 128, 16, 64, 64))
+    rng = np.random.default_rng(10)
+    A = rng.integers(-8, 9, (257, 300)).astype(np.float32)
+    B = rng.integers(-8, 9, (300, 129)).astype(np.float32)
+    assert np.array_equal(run_sgemm_f32(lib, A, B), (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32))
+    Bf = rng.standard_normal((96, 77)).astype(np.float32)
+    assert np.array_equal(run_sgemm_f32(lib, np.eye(96, dtype=np.float32), Bf), Bf)
+    E = np.zeros((20, 96), np.float32)
+    E[3, 90] = 1
+    want = np.zeros((20, 77), np.float32)
+    want[3] = Bf[90]
+    assert np.array_equal(run_sgemm_f32(lib, E, Bf), want)
+    for f in sorted(glob.glob(os.path.join(GOLDEN, "gemm_f32_*.npz"))):
+        d = np.load(f)
+        assert normwise(run_sgemm_f32(lib, d["A"], d["B"]), d["C64"]) < TOL32, f
+    t = torch.zeros((64, 64), dtype=torch.float32, device="cuda:0")
+    assert lib.gemm(t.data_ptr(), t.data_ptr(), t.data_ptr(), 62, 64, 64, 62, 64, 64, check=False) == \
+        HELIX_ERR_INVALID_VALUE   # lda % 4
+
+
+def test_sgemm_f32_config1_and_large_k():
+    """config 1 (1024^3, U[-1,1)) against the x86 path's result, and K = 8192 where FP32 summation order
+    matters most (sequential-k CPU vs MFMA order)."""
+    lib = load(b32.sgemm_library(256, 128, 16, 128, 64))
+    A = seeded_inputs.uniform_pm1((1024, 1024), seeded_inputs.SEED_A)
+    B = seeded_inputs.uniform_pm1((1024, 1024), seeded_inputs.SEED_B)
+    want = O.x86_sch_gemm(A, B, (4, 1, 8, 16, 3, 2, 4), nthreads=8)
+    assert normwise(run_sgemm_f32(lib, A, B), want) < TOL32
+    A = seeded_inputs.normal((64, 8192), 0.1, seeded_inputs.SEED_A)
+    B = seeded_inputs.normal((8192, 96), 0.1, seeded_inputs.SEED_B)
+    assert normwise(run_sgemm_f32(lib, A, B), O.sgemm_seqk(A, B)) < TOL32
+
+
+def test_conv_f32_vs_oracle():
+    for cfg in [(128, 128, 16, 64, 64), (32, 32, 8, 32, 32), (64, 64, 32, 32, 32)]:
+        lib = load(b32.sgemm_library(*cfg))
+        for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS + [(2, 8, 8, 4, 8, 3, 3, 1, 1)]:
+            x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW, dtype=np.float32)
+            got = run_conv(lib, x, w, stride, pad, torch.float32)
+            want = O.conv2d_nhwc(x, w, stride, pad)
+            assert not np.isnan(got).any(), (cfg, batch, H, W, IC, OC, kH, kW, stride, pad)
+            assert normwise(got, want) < TOL32, (cfg, batch, H, W, IC, OC, kH, kW, stride, pad)
+
+
+@pytest.mark.parametrize("name", ["gemv_fp32", "gemv_fp32_splitK"])
+def test_gemv_f32_vs_oracle(name):
+    lib = load(b32.kernel_library(name))
+    for M in (1, 3, 4, 16, 17):
+        for (N, K) in [(128, 256), (1000, 1028), (4096, 2048), (9001, 4)]:
+            x = seeded_inputs.normal((M, K), 1.0, seeded_inputs.SEED_A)
+            W = seeded_inputs.normal((K, N), 0.02, seeded_inputs.SEED_B)
+            dx, dW = dev(x), dev(W.T)
+            dy = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda:0")
+            wsb = lib.workspace_bytes(M, N, K)
+            ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda:0")
+            lib.gemm(dx.data_ptr(), dW.data_ptr(), dy.data_ptr(), M, N, K, K, K, N, ws.data_ptr(), wsb)
+            torch.cuda.synchronize()
+            got = dy.cpu().numpy()
+            assert not np.isnan(got).any(), (M, N, K)
+            assert normwise(got, O.sgemm_seqk(x, W)) < TOL32, (M, N, K)
+
+
+# ---------------------------------------------------------------------------------------------
+# timing entry points and the host loop
+# ---------------------------------------------------------------------------------------------
+def test_bench_entry_points_return_sane_times():
+    lib = load(b16.kernel_library("gemm", 2, 128, 128, 64, 64, 64))
+    mn, avg, mx = lib.bench(1024, 1024, 1024, warmup=2, iters=5, outer=2)
+    assert 0 < mn <= avg <= mx < 1e-2
+    mn, avg, mx = lib.bench_conv(2, 64, 14, 14, 64, 3, 3, 1, 1, warmup=2, iters=5, outer=1)
+    assert 0 < mn <= avg <= mx < 1e-2
+    gv = load(b16.kernel_library("gemv"))
+    mn, avg, mx = gv.bench(4, 4096, 4096, warmup=2, iters=5, outer=1, rotate_bytes=256 << 20)
+    assert 0 < mn < 1e-2
+    A = torch.zeros((512, 512), dtype=torch.float16, device="cuda:0")
+    t = lib.gemm_timed(A.data_ptr(), A.data_ptr(), A.data_ptr(), 512, 512, 512, 512, 512, 512, warmup=1, iters=3)
+    assert 0 < t < 1e-2
+
+
+def test_profile_select_run_loop(tmp_path, monkeypatch):
+    """build -> profile -> cost-model select -> run, on a handful of configurations."""
+    from utils import helix_runtime
+    from MI355X_FP16 import profile_MI355X_FP16 as p16
+    from MI355X_FP16 import MI355X_FP16_gemm as g16
+    from MI355X_FP16 import MI355X_FP16_conv as c16
+    keys = [(2, 256, 256, 128, 128, 0, 64), (2, 128, 128, 64, 64, 0, 64), (2, 64, 64, 32, 32, 1, 64),
+            (0, 1, 128, 0, 0, 0, 0), (0, 16, 128, 0, 0, 0, 0)]
+    prof = {k: p16.time_config(k, warmup=1, iters=3) for k in keys}
+    assert all(0 < v < 1 for v in prof.values())
+    cost, tflops = g16.get_MI355X_FP16_gemm_Helix_result(prof, 2048, 2048, 2048)
+    assert cost > 0 and 10 < tflops < 2600
+    big_or_gemv = {k: v for k, v in prof.items() if k[0] == 0 or k[1] == 256}
+    assert g16.cost_model(big_or_gemv, 1, 28672, 8192)[0] == 0          # decode shape goes to the GEMV kernel
+    assert g16.cost_model(prof, 8192, 8192, 8192) == (2, 256, 256, 128, 128, 0, 64)
+    cost, tflops = c16.get_MI355X_FP16_conv_Helix_result(prof, 32, 64, 56, 56, 64, 3, 3, 1, 1)
+    assert cost > 0 and tflops > 1
+    ms, tf, key = g16.get_MI355X_FP16_gemm_Oracle_result(prof, 1024, 1024, 1024)
+    assert key in prof and tf > 1

@@ -1,0 +1,244 @@
+"""CPU-only tests of the host side: template-space enumeration, artifact naming, cost models, dict and
+stdout formats, dispatcher tables, and that every built library exports the whole C ABI."""
+import ctypes
+import glob
+import math
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+from utils import hip_ctypes, helix_runtime, roofline
+from utils import get_benchmark_shape_list as shapes
+from MI355X_FP16 import build_MI355X_FP16 as b16
+from MI355X_FP16 import profile_MI355X_FP16 as p16
+from MI355X_FP16 import MI355X_FP16_gemm as g16
+from MI355X_FP16 import MI355X_FP16_conv as c16
+from MI355X_FP16 import benchmark_MI355X_FP16_performance_comparison as cmp16
+from MI355X_FP32 import build_MI355X_FP32 as b32
+from MI355X_FP32 import profile_MI355X_FP32 as p32
+from MI355X_FP32 import MI355X_FP32_gemm as g32
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- enumeration ----------------------------------------------------------------------------------
+def test_fp16_reference_validity_rules():
+    # the four rules of build_Ampere_FP16.py:30-39 keep their meaning
+    assert not b16.is_valid_config(4, 4, 128, 128, 32, 32)            # 4x4 scale
+    assert not b16.is_valid_config(4, 1, 512, 128, 128, 128)          # block > 256
+    assert not b16.is_valid_config(1, 1, 16, 128, 16, 128)            # wave aspect 8x
+    assert not b16.is_valid_config(1, 4, 16, 256, 16, 64)             # block aspect 16x
+    assert b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 2)
+    # gfx950 resource rules
+    assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 128, 3)  # 3 x 512 x 128 x 2 B > 160 KiB of LDS
+
+
+def test_fp16_template_space():
+    cfgs = list(b16.iter_configs())
+    assert len(cfgs) == 112 and len(set(cfgs)) == 112
+    for (st, br, bc, wr, wc, bk) in cfgs:
+        assert br % wr == 0 and bc % wc == 0 and br <= 256 and bc <= 256
+        assert st * (br + bc) * bk * 2 <= 160 * 1024
+        threads = 64 * (br // wr) * (bc // wc)
+        assert threads <= 512 and (br * bk // 8) % threads == 0 and (bc * bk // 8) % threads == 0
+    assert (2, 256, 256, 128, 128, 64) in cfgs
+    keys = p16.all_keys()
+    assert len(keys) == 2 * 112 + 6
+    assert all(len(k) == 7 for k in keys)
+    assert sum(1 for k in keys if k[0] == 0) == 6   # GEMV rows are tagged by a zero first field
+
+
+def test_fp16_library_names():
+    assert b16.library_for_key((2, 256, 128, 64, 64, 0, 32)).endswith("build/bin_fp16/libgemm_2_256_128_64_64_32.so")
+    assert b16.library_for_key((2, 256, 128, 64, 64, 1, 32)).endswith("build/bin_fp16/libgemm_splitK_2_256_128_64_64_32.so")
+    assert b16.library_for_key((0, 1, 128, 0, 0, 0, 0)).endswith("build/bin_fp16/libgemv.so")
+    assert b16.library_for_key((0, 16, 128, 0, 0, 1, 0)).endswith("build/bin_fp16/libgemv_splitK.so")
+    src, out, defines = b16.compile_job("gemm_splitK", 2, 128, 64, 64, 32, 64)
+    assert src.endswith("src_template/MI355X_FP16/gemm.hip")
+    assert defines == {"SPLIT_K": 2, "LDS_STAGES": 2, "BLOCK_ROWS": 128, "BLOCK_COLS": 64, "WAVE_ROWS": 64,
+                       "WAVE_COLS": 32, "BLOCK_K": 64}
+    cmd = helix_runtime.compile_command(src, out, defines)
+    assert "--offload-arch=gfx950" in cmd and "-DBLOCK_ROWS=128" in cmd and "-shared" in cmd
+    assert "-packed-fp32-ops" in cmd
+
+
+def test_fp32_template_space():
+    cfgs = list(b32.iter_configs())
+    assert len(cfgs) == 143 and len(set(cfgs)) == 143
+    for (BM, BN, BK, WM, WN) in cfgs:
+        assert BM % WM == 0 and BN % WN == 0 and 32 <= BM <= 256 and 32 <= BN <= 256
+        assert 64 * (BM // WM) * (BN // WN) <= 512
+    keys = p32.all_keys()
+    assert len(keys) == 143 + 6 and all(len(k) == 8 for k in keys)
+    assert b32.library_for_key((128, 64, 16, 64, 32, 2, 4, 4)).endswith("build/bin_fp32/libsgemm_128_64_16_64_32.so")
+    assert b32.library_for_key((4, 128, 0, 0, 0, 0, 4, 4)).endswith("build/bin_fp32/libgemv_fp32.so")
+    assert b32.library_for_key((4, 128, 0, 0, 0, 1, 4, 4)).endswith("build/bin_fp32/libgemv_fp32_splitK.so")
+
+
+# ---- cost model ---------------------------------------------------------------------------------------
+def test_fp16_cost_model_hand_cases():
+    K = p16.PROFILE_K
+    # 4096^2 outputs: 128x128 tiles -> 1024 blocks -> 4 rounds x 1.0; 256x128 -> 512 blocks -> 2 rounds x 1.8
+    d = {(2, 128, 128, 64, 64, 0, 64): 1.0, (2, 256, 128, 64, 64, 0, 64): 1.8}
+    assert g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 4096, 4096, K) == pytest.approx(4.0)
+    assert g16.config_cost((2, 256, 128, 64, 64, 0, 64), 1.8, 4096, 4096, K) == pytest.approx(3.6)
+    assert g16.cost_model(d, 4096, 4096, K) == (2, 256, 128, 64, 64, 0, 64)
+    # the quantisation is what makes the small tile win on a small problem: 300x300 -> 9 vs 4 blocks, one round each
+    assert g16.cost_model(d, 300, 300, K) == (2, 128, 128, 64, 64, 0, 64)
+    # round time scales with K
+    assert g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 4096, 4096, K // 2) == pytest.approx(2.0)
+    # split-K doubles the blocks (reference: * (k[5] + 1)) and halves the K walk
+    c0 = g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 128, 128, 8192)
+    c1 = g16.config_cost((2, 128, 128, 64, 64, 1, 64), 1.0, 128, 128, 8192)
+    assert c1 < c0
+    assert g16.config_cost((2, 128, 128, 64, 64, 1, 64), 1.0, 4096 * 4, 4096, K) > \
+        g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 4096 * 4, 4096, K) * 0.99
+    # GEMV rows: blocks = ceil(small / row tile) * ceil(big / 128), proportional share of a 256-block round
+    gemv = (0, 4, 128, 0, 0, 0, 0)
+    assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 256, K) == pytest.approx(2.56e-3)
+    assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 128, K) == pytest.approx(1.28e-3)
+    assert g16.config_cost(gemv, 2.56e-3, 128 * 256, 3, K) == pytest.approx(2.56e-3)      # operands swap
+    assert g16.config_cost(gemv, 2.56e-3, 16, 128 * 256, K) == pytest.approx(4 * 2.56e-3)
+    assert g16.config_cost(gemv, 1e-9, 1, 128, 512) == g16.GEMV_LAUNCH_FLOOR_S
+    # conv never selects a GEMV row
+    d2 = dict(d)
+    d2[gemv] = 1e-12
+    assert c16.cost_model(d2, 4096, 4096, K)[0] != 0
+    assert g16.cost_model(d2, 4, 4096, K) == gemv
+
+
+def test_static_cost_models():
+    d = {(2, 128, 128, 64, 64, 0, 64): 1.0, (2, 64, 64, 64, 64, 0, 64): 0.4, (2, 256, 128, 64, 64, 0, 64): 1.8,
+         (0, 1, 128, 0, 0, 0, 0): 1e-9}
+    assert cmp16.cost_model_static1(d, 4096, 4096, 4096) == (2, 64, 64, 64, 64, 0, 64)     # only block == wave tile
+    assert cmp16.cost_model_static2(d, 64, 64, 64) == (2, 256, 128, 64, 64, 0, 64)         # best time per tile area
+
+
+def test_fp32_cost_model_hand_cases():
+    K = p32.PROFILE_K
+    d = {(128, 128, 16, 64, 64, 2, 4, 4): 1.0, (256, 128, 16, 128, 64, 2, 4, 4): 1.8}
+    assert g32.cost_model(d, 4096, 4096, K) == (256, 128, 16, 128, 64, 2, 4, 4)
+    assert g32.cost_model(d, 300, 300, K) == (128, 128, 16, 64, 64, 2, 4, 4)
+    assert g32.config_cost((128, 128, 16, 64, 64, 2, 4, 4), 1.0, 4096, 4096, 2 * K) == pytest.approx(8.0)
+
+
+def test_padded_k():
+    assert g16.padded_k(770) == 776 and g16.padded_k(768) == 768 and g16.padded_k(1) == 8
+
+
+# ---- formats --------------------------------------------------------------------------------------------
+def test_reference_stdout_line_token():
+    line = helix_runtime.reference_line(256, 128, 4096, 1.25e-5, 1.5e-5, 2.0e-5)
+    assert float(line.split()[-8]) == pytest.approx(1.5e-5)      # what profile_Ampere_FP16.py:38 parses
+    assert line.startswith("M N K =    256    128   4096, Time =")
+    assert line.endswith("Tflops")
+
+
+def test_prof_dict_roundtrip(tmp_path, monkeypatch):
+    monkeypatch.setattr(helix_runtime, "root_path", str(tmp_path))
+    d = {(2, 128, 128, 64, 64, 0, 64): 1.5e-5, (0, 1, 128, 0, 0, 0, 0): float("inf")}
+    helix_runtime.write_prof_dict("MI355X_FP16", d)
+    text = open(tmp_path / "build" / "prof_dict" / "MI355X_FP16_cost_model.dict").read()
+    assert "\n" not in text and text.startswith("{(2, 128, 128, 64, 64, 0, 64): 1.5e-05")
+    # `inf` is not a Python literal: the reader evaluates the line exactly as the reference does
+    # (eval(lines[0]), benchmark_Ampere_FP16_gemm.py:10-12), with inf defined
+    assert "inf" in text
+    assert helix_runtime.read_prof_dict("MI355X_FP16") == d
+
+
+def test_shape_lists():
+    g = shapes.get_gemm_op_MNKList()
+    assert len(g) == 60 * 16 + 8 * 10 and g[0] == (2, 1024, 1024) and g[15] == (2, 4096, 11008)
+    bert, llama, gpt2 = shapes.get_llm_opset_MNKList()
+    assert len(bert) == 60 * 73 and len(llama) == 60 * 4 and len(gpt2) == 60 * 96
+    bb = shapes.get_baseline_bert_MNKList()
+    assert len(bb) == 49 and bb[-1] == (4000, 2300, 770) and bb[0] == (4096, 2304, 768)
+    flops = sum(2 * m * n * k for (m, n, k) in bb)
+    assert flops == pytest.approx(695.8e9 + 14.17e9, rel=1e-3)
+    conv = shapes.get_baseline_conv_shape_list()
+    assert len(conv) == 6 and conv[0] == (32, 64, 56, 56, 64, 3, 3, 1, 1)
+    want = [7.40, 3.29, 7.40, 7.40, 7.40, 6.58]
+    for s, w in zip(conv, want):
+        assert roofline.conv_flops(*s) / 1e9 == pytest.approx(w, abs=0.01)
+
+
+def test_roofline_constants():
+    assert roofline.FP16_MFMA_FLOPS == 2516.6e12 and roofline.FP32_MFMA_FLOPS == 157.3e12
+    assert roofline.HBM_BYTES_PER_S == 8.0e12 and roofline.NUM_CU == 256
+    assert roofline.gemm_bytes(1, 4096, 4096, 2) / 1e6 == pytest.approx(33.6, abs=0.05)
+    assert roofline.gemm_bytes(1, 28672, 8192, 2) / 1e6 == pytest.approx(469.8, abs=0.1)
+    assert roofline.gemm_flops(8192, 8192, 8192) / roofline.FP16_MFMA_FLOPS * 1e6 == pytest.approx(436.9, abs=0.1)
+
+
+# ---- dispatchers --------------------------------------------------------------------------------------------
+def test_dispatch_tables_resolve():
+    import _dispatch
+    import build_template, profile_template, changed_profile, runtime_cost, benchmark_op_level_eval, \
+        benchmark_model_level_eval
+    for rows in build_template.func_dict.values():
+        for row in rows:
+            assert callable(_dispatch.resolve(row))
+    for table in (profile_template.func_dict, changed_profile.func_dict, runtime_cost.func_dict,
+                  benchmark_op_level_eval.func_dict, benchmark_model_level_eval.func_dict):
+        for row in table.values():
+            assert callable(_dispatch.resolve(row))
+
+
+def test_cli_unsupported_combination_message():
+    env = dict(os.environ, PYTHONPATH=os.path.join(ROOT, "helix_amd", "scripts"))
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "helix_amd", "scripts", "benchmark_op_level_eval.py"), "-o",
+                          "GEMM", "-b", "MI355X_FP16", "-s", "rocblas"], capture_output=True, text=True, env=env, cwd=ROOT)
+    assert out.returncode == 0 and out.stdout.strip() == "GEMM MI355X_FP16 rocblas is not supported"
+
+
+# ---- C ABI ------------------------------------------------------------------------------------------------------
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "helix_abi.h")).read()
+    return sorted(set(re.findall(r"^(?:int|size_t)\s+(helix_\w+)\s*\(", text, flags=re.M)))
+
+
+def test_header_matches_binding():
+    assert _declared_symbols() == sorted(hip_ctypes.ABI_SYMBOLS)
+
+
+def _built_libraries():
+    return sorted(glob.glob(os.path.join(ROOT, "build", "bin_fp16", "*.so")) +
+                  glob.glob(os.path.join(ROOT, "build", "bin_fp32", "*.so")))
+
+
+def test_every_built_library_exports_the_whole_abi():
+    libs = _built_libraries()
+    if not libs:
+        pytest.skip("kernel libraries are not built (run __graft_entry__.build())")
+    want = set(_declared_symbols())
+    # dlopen + dlsym only; no compute without a GPU.  A sample keeps this fast: every family, every 7th gemm
+    sample = [p for p in libs if "gemv" in p] + libs[::7]
+    for path in sample:
+        assert set(hip_ctypes.exported_symbols(path)) == want, path
+        info = hip_ctypes.HelixLib(path).info()
+        assert info["arch"] == "gfx950" and info["family"] in ("gemm_f16", "gemv_f16", "sgemm_f32", "gemv_f32")
+
+
+def test_all_expected_libraries_are_built():
+    if not _built_libraries():
+        pytest.skip("kernel libraries are not built (run __graft_entry__.build())")
+    missing = [out for (_, out, _) in b16.build_jobs() + b32.build_jobs() if not os.path.exists(out)]
+    assert not missing, missing[:5]
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(FileNotFoundError):
+        hip_ctypes.HelixLib(str(tmp_path / "libgemm_nope.so"))
+
+
+def test_info_matches_file_name():
+    path = b16.kernel_library("gemm", 2, 256, 128, 64, 64, 32)
+    if not os.path.exists(path):
+        pytest.skip("kernel libraries are not built")
+    info = hip_ctypes.HelixLib(path).info()
+    assert (info["lds_stages"], info["block_rows"], info["block_cols"], info["wave_rows"], info["wave_cols"],
+            info["block_k"], info["split_k"]) == (2, 256, 128, 64, 64, 32, 1)
+    assert info["threads"] == 64 * 4 * 2 and info["lds_bytes"] == 2 * (256 + 128) * 32 * 2
