@@ -19,9 +19,11 @@
 // Kernel structure
 //   * one wave64 computes (WAVE_ROWS/32) x (WAVE_COLS/32) v_mfma_f32_32x32x16_f16 tiles; per 16-wide
 //     k step it reads one 16-byte fragment per 32 rows of A and of B from LDS (ds_read_b128).
-//   * global -> LDS goes through buffer loads (128-bit per lane, hardware bounds checking zero-fills
-//     rows beyond M / N) into registers and ds_write_b128; the loads for stage s+1 are issued before
-//     the MFMAs of stage s and written to LDS after them, one barrier per stage.
+//   * global -> LDS uses gfx950's 128-bit direct-to-LDS buffer loads (DIRECT_TO_LDS=1, default): no
+//     staging registers, no ds_write; hardware bounds checking zero-fills rows beyond M / N and the K
+//     tail.  The copy of tile t+1 is issued after tile t's fragments are read and lands while tile t's
+//     MFMAs run; one wait + barrier per tile.  DIRECT_TO_LDS=0 keeps the register-staged variant
+//     (buffer_load -> VGPR -> ds_write_b128).
 //   * LDS rows are BLOCK_K halves; 16-byte chunk c of row r is stored at chunk (c ^ key(r)), with
 //     key(r) = (r / rows_per_256B) mod chunks_per_row, so that 16 consecutive rows of one chunk column
 //     land in 16 different 16-byte bank groups (64 banks x 4 B): fragment reads and tile writes are
@@ -57,6 +59,9 @@
 #endif
 #ifndef GROUP_ROWS
 #define GROUP_ROWS 8
+#endif
+#ifndef DIRECT_TO_LDS
+#define DIRECT_TO_LDS 1
 #endif
 
 namespace {
@@ -109,11 +114,21 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
+constexpr int OOB_OFFSET = 0x7fffffff;  // byte offset beyond any buffer: the load returns zeros
+constexpr int KSTEPS = BK / 16;         // MFMA k-steps per K tile
+typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
+
+// s_waitcnt vmcnt(0): every outstanding buffer load of this wave (also the direct-to-LDS ones) has landed
+__device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 __device__ __forceinline__ intx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) {
     return __builtin_bit_cast(intx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
 }
 
-template <bool CONV>
+// The tile parameters appear as (otherwise unused) template arguments so that every configuration's
+// kernel has its own symbol name and a profiler lists configurations separately.
+template <bool CONV, int T_STAGES = STAGES, int T_BM = BM, int T_BN = BN, int T_WM = WM, int T_WN = WN, int T_BK = BK,
+          int T_SPLITK = SPLITK>
 __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
@@ -151,19 +166,16 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     }
 
     // ---- per-thread copy geometry ---------------------------------------------------------------
-    const int kc = tid % KCH;          // 16-byte chunk within a tile row (same for every iteration)
-    const int r0 = tid / KCH;          // first tile row this thread copies
-    int lds_wr_a[A_ITERS], lds_wr_b[B_ITERS];
+    // Copy slot c = tid + i*NTHREADS of a tile lands at LDS byte c*16 (so one wave-wide copy instruction
+    // fills 1 KiB of consecutive LDS, which is what a direct-to-LDS load requires); it holds row r = c / KCH
+    // and, because of the swizzle, global chunk g = (c % KCH) ^ key(r) of that row.
+    const int cpos = tid % KCH;
+    const int r0 = tid / KCH;
+    int gch_a[A_ITERS], gch_b[B_ITERS];    // global 16-byte chunk index within the K tile
 #pragma unroll
-    for (int i = 0; i < A_ITERS; i++) {
-        const int r = r0 + i * ROWS_PER_ITER;
-        lds_wr_a[i] = r * ROW_BYTES + ((kc ^ swz_key(r)) << 4);
-    }
+    for (int i = 0; i < A_ITERS; i++) gch_a[i] = cpos ^ swz_key(r0 + i * ROWS_PER_ITER);
 #pragma unroll
-    for (int i = 0; i < B_ITERS; i++) {
-        const int r = r0 + i * ROWS_PER_ITER;
-        lds_wr_b[i] = A_STAGE_BYTES + r * ROW_BYTES + ((kc ^ swz_key(r)) << 4);
-    }
+    for (int i = 0; i < B_ITERS; i++) gch_b[i] = cpos ^ swz_key(r0 + i * ROWS_PER_ITER);
 
     // B operand: rows n0.. of an N x K matrix
     const int rows_b = (p.N - n0) < BN ? (p.N - n0) : BN;
@@ -171,7 +183,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     const unsigned bytesB = (unsigned)(((size_t)(rows_b - 1) * p.ldb + p.K) * 2);
     int voff_b[B_ITERS];
 #pragma unroll
-    for (int i = 0; i < B_ITERS; i++) voff_b[i] = ((r0 + i * ROWS_PER_ITER) * p.ldb + kc * 8) * 2;
+    for (int i = 0; i < B_ITERS; i++) voff_b[i] = ((r0 + i * ROWS_PER_ITER) * p.ldb + gch_b[i] * 8) * 2;
 
     // A operand
     const half_t* baseA = nullptr;
@@ -183,7 +195,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         baseA = p.A + (size_t)m0 * p.lda;
         bytesA = (unsigned)(((size_t)(rows_a - 1) * p.lda + p.K) * 2);
 #pragma unroll
-        for (int i = 0; i < A_ITERS; i++) voff_a[i] = ((r0 + i * ROWS_PER_ITER) * p.lda + kc * 8) * 2;
+        for (int i = 0; i < A_ITERS; i++) voff_a[i] = ((r0 + i * ROWS_PER_ITER) * p.lda + gch_a[i] * 8) * 2;
     } else {
         baseA = p.A;
         bytesA = p.a_bytes;
@@ -200,46 +212,68 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         }
     }
 
-    intx4 stage_a[A_ITERS], stage_b[B_ITERS];
-
-    auto load_global = [&](int k0) {
-        const bool tail = (k0 + BK > p.K);
-        const bool dead = tail && (k0 + kc * 8 >= p.K);  // chunk lies beyond K: contributes zero
-        __amdgpu_buffer_rsrc_t rb = make_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u);
-#pragma unroll
-        for (int i = 0; i < B_ITERS; i++) {
-            stage_b[i] = buf_load16(rb, dead ? (int)0x7fffffff : voff_b[i]);
-        }
+    // Byte offset (relative to the operand's buffer descriptor) of copy slot i for the K tile at k0, or
+    // OOB_OFFSET when the slot must read zeros (beyond K, conv padding, rows beyond M).
+    auto a_offset = [&](int i, int k0, bool tail) -> int {
         if (!CONV) {
-            __amdgpu_buffer_rsrc_t ra = make_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
-#pragma unroll
-            for (int i = 0; i < A_ITERS; i++) {
-                stage_a[i] = buf_load16(ra, dead ? (int)0x7fffffff : voff_a[i]);
-            }
+            return (tail && k0 + gch_a[i] * 8 >= p.K) ? OOB_OFFSET : voff_a[i];
         } else {
-            __amdgpu_buffer_rsrc_t ra = make_rsrc(baseA, bytesA);
-            const int k = k0 + kc * 8;       // k = (kh*kW + kw)*IC + c, 8 consecutive c per chunk
+            const int k = k0 + gch_a[i] * 8;  // k = (kh*kW + kw)*IC + c, 8 consecutive c per chunk
             const int c = k % p.g.IC;
             const int t = k / p.g.IC;
             const int kw = t % p.g.kW;
             const int kh = t / p.g.kW;
-#pragma unroll
-            for (int i = 0; i < A_ITERS; i++) {
-                const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
-                const bool ok = !dead && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W;
-                const int off = ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 2;
-                stage_a[i] = buf_load16(ra, ok ? off : (int)0x7fffffff);
-            }
+            const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
+            const bool ok = k < p.K && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W;
+            return ok ? ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 2 : OOB_OFFSET;
         }
     };
-
-    auto store_lds = [&](int stage) {
-        unsigned char* base = smem + stage * STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < A_ITERS; i++) *(intx4*)(base + lds_wr_a[i]) = stage_a[i];
-#pragma unroll
-        for (int i = 0; i < B_ITERS; i++) *(intx4*)(base + lds_wr_b[i]) = stage_b[i];
+    auto b_offset = [&](int i, int k0, bool tail) -> int {
+        return (tail && k0 + gch_b[i] * 8 >= p.K) ? OOB_OFFSET : voff_b[i];
     };
+
+#if DIRECT_TO_LDS
+    // global -> LDS without passing through registers: each wave-wide load deposits 64 x 16 bytes at a
+    // wave-uniform LDS address (slot base of the wave) in lane order.
+    auto copy_tile = [&](int stage, int k0) {
+        const bool tail = (k0 + BK > p.K);
+        __amdgpu_buffer_rsrc_t rb = make_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u);
+        __amdgpu_buffer_rsrc_t ra = CONV ? make_rsrc(baseA, bytesA) : make_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
+        // (pointer arithmetic is done on the generic pointer, the LDS-qualified cast comes last)
+        unsigned char* sa = smem + stage * STAGE_BYTES + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) {
+            const int off = a_offset(i, k0, tail);
+            lds_ptr_t dst = (lds_ptr_t)(sa + i * NTHREADS * 16);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, off, 0, 0, 0);
+        }
+        unsigned char* sb = sa + A_STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < B_ITERS; i++) {
+            const int off = b_offset(i, k0, tail);
+            lds_ptr_t dst = (lds_ptr_t)(sb + i * NTHREADS * 16);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, off, 0, 0, 0);
+        }
+    };
+#else
+    intx4 stage_a[A_ITERS], stage_b[B_ITERS];
+    auto load_global = [&](int k0) {
+        const bool tail = (k0 + BK > p.K);
+        __amdgpu_buffer_rsrc_t rb = make_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u);
+        __amdgpu_buffer_rsrc_t ra = CONV ? make_rsrc(baseA, bytesA) : make_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
+#pragma unroll
+        for (int i = 0; i < B_ITERS; i++) stage_b[i] = buf_load16(rb, b_offset(i, k0, tail));
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) stage_a[i] = buf_load16(ra, a_offset(i, k0, tail));
+    };
+    auto store_lds = [&](int stage) {
+        unsigned char* base = smem + stage * STAGE_BYTES + tid * 16;
+#pragma unroll
+        for (int i = 0; i < A_ITERS; i++) *(intx4*)(base + i * NTHREADS * 16) = stage_a[i];
+#pragma unroll
+        for (int i = 0; i < B_ITERS; i++) *(intx4*)(base + A_STAGE_BYTES + i * NTHREADS * 16) = stage_b[i];
+    };
+#endif
 
     // ---- fragment read geometry -----------------------------------------------------------------
     // MFMA 32x32x16: lane l supplies row (l % 32), k = 8*(l/32) .. +7 of both operands.
@@ -247,6 +281,12 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     const int a_row = wave_m * WM + frow;
     const int b_row = wave_n * WN + frow;
     const int a_rd = a_row * ROW_BYTES, b_rd = A_STAGE_BYTES + b_row * ROW_BYTES;
+    auto read_a = [&](const unsigned char* sb, int s, int i) -> half8 {
+        return *(const half8*)(sb + a_rd + i * 32 * ROW_BYTES + (((s * 2 + fhalf) ^ swz_key(a_row + i * 32)) << 4));
+    };
+    auto read_b = [&](const unsigned char* sb, int s, int j) -> half8 {
+        return *(const half8*)(sb + b_rd + j * 32 * ROW_BYTES + (((s * 2 + fhalf) ^ swz_key(b_row + j * 32)) << 4));
+    };
 
     floatx16 acc[TM][TN];
 #pragma unroll
@@ -257,6 +297,69 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
 
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
+
+#if DIRECT_TO_LDS
+    // Two LDS stages.  Per K tile: read the fragments of k-steps 1.. of the current stage, start the
+    // direct-to-LDS copy of the next tile into the other stage, run the MFMAs of all but the last
+    // k-step, wait for the copy and synchronise, read the first k-step's fragments of the next tile, and
+    // run the last k-step's MFMAs underneath those reads.
+    if (ktiles > 0) copy_tile(0, k_begin);
+    wait_vmcnt0();
+    __syncthreads();
+    half8 a0[TM], b0[TN];
+    if (ktiles > 0) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) a0[i] = read_a(smem, 0, i);
+#pragma unroll
+        for (int j = 0; j < TN; j++) b0[j] = read_b(smem, 0, j);
+    }
+    for (int kt = 0; kt < ktiles; kt++) {
+        const int cur = kt & 1;
+        const bool more = (kt + 1 < ktiles);
+        const unsigned char* sb = smem + cur * STAGE_BYTES;
+        half8 af[KSTEPS][TM], bf[KSTEPS][TN];
+#pragma unroll
+        for (int s = 1; s < KSTEPS; s++) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) af[s][i] = read_a(sb, s, i);
+#pragma unroll
+            for (int j = 0; j < TN; j++) bf[s][j] = read_b(sb, s, j);
+        }
+        if (more) copy_tile(cur ^ 1, k_begin + (kt + 1) * BK);
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0[i], b0[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+        for (int s = 1; s < KSTEPS - 1; s++)
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[s][i], bf[s][j], acc[i][j], 0, 0, 0);
+        // keep the instruction scheduler from hoisting the wait and barrier above the MFMAs that hide the copy
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vmcnt0();
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (more) {
+            const unsigned char* sn = smem + (cur ^ 1) * STAGE_BYTES;
+#pragma unroll
+            for (int i = 0; i < TM; i++) a0[i] = read_a(sn, 0, i);
+#pragma unroll
+            for (int j = 0; j < TN; j++) b0[j] = read_b(sn, 0, j);
+        }
+        if (KSTEPS > 1) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[KSTEPS - 1][i], bf[KSTEPS - 1][j], acc[i][j],
+                                                                       0, 0, 0);
+        }
+    }
+#else
     if (ktiles > 0) {
         load_global(k_begin);
         store_lds(0);
@@ -270,15 +373,12 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 
         const unsigned char* sb = smem + cur * STAGE_BYTES;
 #pragma unroll
-        for (int s = 0; s < BK / 16; s++) {
+        for (int s = 0; s < KSTEPS; s++) {
             half8 af[TM], bf[TN];
-            const int ch = s * 2 + fhalf;
 #pragma unroll
-            for (int i = 0; i < TM; i++)
-                af[i] = *(const half8*)(sb + a_rd + i * 32 * ROW_BYTES + ((ch ^ swz_key(a_row + i * 32)) << 4));
+            for (int i = 0; i < TM; i++) af[i] = read_a(sb, s, i);
 #pragma unroll
-            for (int j = 0; j < TN; j++)
-                bf[j] = *(const half8*)(sb + b_rd + j * 32 * ROW_BYTES + ((ch ^ swz_key(b_row + j * 32)) << 4));
+            for (int j = 0; j < TN; j++) bf[j] = read_b(sb, s, j);
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -289,6 +389,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         if (more) store_lds(cur ^ 1);
         __syncthreads();
     }
+#endif
 
     // ---- epilogue: lane l holds column (l % 32); rows 8*(v/4) + 4*(l/32) + (v%4), v = 0..15 -------
     const int col_l = lane & 31, row_l = (lane >> 5) * 4;

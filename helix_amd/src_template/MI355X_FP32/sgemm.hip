@@ -91,7 +91,9 @@ __device__ __forceinline__ floatx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff
 
 constexpr int OOB = 0x7fffffff;  // byte offset beyond any buffer: the load returns zeros
 
-template <bool CONV>
+// The tile parameters appear as (otherwise unused) template arguments so that every configuration's
+// kernel has its own symbol name and a profiler lists configurations separately.
+template <bool CONV, int T_BM = BM, int T_BN = BN, int T_BK = BK, int T_WM = WAVE_M, int T_WN = WAVE_N>
 __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params p) {
     extern __shared__ __attribute__((aligned(16))) float smem[];
 
