@@ -85,6 +85,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gemv", action="store_true")
+    ap.add_argument("--kernel-config", type=str, default=None,
+                    help="skip the template search and time this configuration, e.g. 2,256,256,64,128,0,64")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one 1 GiB device copy (a reference point for HBM traffic counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (every GPU box has one GPU); "
@@ -106,7 +110,10 @@ def main():
 
     # ---- autotune: full template search on this shape ------------------------------------------------
     t0 = time.perf_counter()
-    best, best_t, tried = autotune(all_keys(), M, N, K)
+    if args.kernel_config:
+        best, tried = tuple(int(x) for x in args.kernel_config.split(",")), 0
+    else:
+        best, best_t, tried = autotune(all_keys(), M, N, K)
     autotune_s = time.perf_counter() - t0
     lib = load(library_for_key(best))
 
@@ -121,6 +128,13 @@ def main():
 
     def step():
         lib.gemm(A.data_ptr(), Bt.data_ptr(), C.data_ptr(), M, N, K, K, K, N, ws.data_ptr(), wsb, stream)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()

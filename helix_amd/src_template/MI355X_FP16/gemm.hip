@@ -89,7 +89,13 @@ static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is built from 32x32 MFMA 
 static_assert(BK % 16 == 0 && (KCH & (KCH - 1)) == 0 && KCH >= 2, "BLOCK_K must be 16 * 2^n");
 static_assert(NTHREADS <= 1024 && NTHREADS % KCH == 0, "bad thread count");
 static_assert((BM * KCH) % NTHREADS == 0 && (BN * KCH) % NTHREADS == 0, "tile copy must divide evenly");
-static_assert(STAGES == 2, "this revision implements the two-stage ring");
+#if DIRECT_TO_LDS
+static_assert(STAGES >= 2 && STAGES <= 4, "LDS ring depth must be 2..4");
+static_assert((BK / 16) % 2 == 0, "BLOCK_K must hold an even number of 16-wide MFMA k-steps");
+static_assert((STAGES - 2) * (A_ITERS + B_ITERS) <= 63, "too many copy instructions in flight for vmcnt");
+#else
+static_assert(STAGES == 2, "the register-staged variant implements the two-stage ring only");
+#endif
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
 static_assert(SPLITK >= 1 && SPLITK <= 8, "SPLIT_K out of range");
 
@@ -118,8 +124,28 @@ constexpr int OOB_OFFSET = 0x7fffffff;  // byte offset beyond any buffer: the lo
 constexpr int KSTEPS = BK / 16;         // MFMA k-steps per K tile
 typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
 
-// s_waitcnt vmcnt(0): every outstanding buffer load of this wave (also the direct-to-LDS ones) has landed
-__device__ __forceinline__ void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+// s_waitcnt vmcnt(N): at most N buffer loads of this wave (also the direct-to-LDS ones) are still in flight
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+// 128-bit buffer descriptor as four dwords: base address (48 bits), stride 0, byte count, raw-buffer flags
+__device__ __forceinline__ intx4 raw_rsrc(const void* base, unsigned bytes) {
+    const unsigned long long a = (unsigned long long)base;
+    intx4 r = {(int)(unsigned)a, (int)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+    return r;
+}
+
+// One 16-byte-per-lane direct-to-LDS buffer load: lane l's data lands at LDS byte (lds_addr + 16*l).
+// lds_addr must be wave-uniform (it is moved into M0); voff is the per-lane byte offset into the buffer.
+__device__ __forceinline__ void dma16(intx4 rsrc, unsigned lds_addr, int voff) {
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc)
+                 : "memory", "m0");
+}
 
 __device__ __forceinline__ intx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) {
     return __builtin_bit_cast(intx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
@@ -134,7 +160,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: lives in a scalar register
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
 
     // ---- workgroup id -> (tile_m, tile_n), XCD-aware ------------------------------------------
@@ -234,27 +260,26 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 
 #if DIRECT_TO_LDS
     // global -> LDS without passing through registers: each wave-wide load deposits 64 x 16 bytes at a
-    // wave-uniform LDS address (slot base of the wave) in lane order.
-    auto copy_tile = [&](int stage, int k0) {
-        const bool tail = (k0 + BK > p.K);
-        __amdgpu_buffer_rsrc_t rb = make_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u);
-        __amdgpu_buffer_rsrc_t ra = CONV ? make_rsrc(baseA, bytesA) : make_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
-        // (pointer arithmetic is done on the generic pointer, the LDS-qualified cast comes last)
-        unsigned char* sa = smem + stage * STAGE_BYTES + wave * 1024;
-#pragma unroll
-        for (int i = 0; i < A_ITERS; i++) {
-            const int off = a_offset(i, k0, tail);
-            lds_ptr_t dst = (lds_ptr_t)(sa + i * NTHREADS * 16);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, off, 0, 0, 0);
-        }
-        unsigned char* sb = sa + A_STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < B_ITERS; i++) {
+    // wave-uniform LDS address (M0) in lane order.  The loads are issued from inline assembly so that
+    // the compiler does not serialise later LDS reads behind them; completion is tracked by hand with
+    // s_waitcnt vmcnt(n) before the workgroup barrier that publishes a stage.
+    const unsigned lds_base = (unsigned)(uintptr_t)(lds_ptr_t)smem;
+    const unsigned lds_wave = lds_base + (unsigned)wave * 1024u;
+    // copy slot `idx` (A slots first, then B slots) of the K tile at k0 into LDS stage `stage`
+    auto copy_slot = [&](int idx, int stage, int k0, bool tail, intx4 ra, intx4 rb) {
+        if (idx < A_ITERS) {
+            const int off = a_offset(idx, k0, tail);
+            dma16(ra, lds_wave + (unsigned)(stage * STAGE_BYTES + idx * NTHREADS * 16), off);
+        } else {
+            const int i = idx - A_ITERS;
             const int off = b_offset(i, k0, tail);
-            lds_ptr_t dst = (lds_ptr_t)(sb + i * NTHREADS * 16);
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, off, 0, 0, 0);
+            dma16(rb, lds_wave + (unsigned)(stage * STAGE_BYTES + A_STAGE_BYTES + i * NTHREADS * 16), off);
         }
     };
+    auto rsrc_a = [&](int k0) -> intx4 {
+        return CONV ? raw_rsrc(baseA, bytesA) : raw_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
+    };
+    auto rsrc_b = [&](int k0) -> intx4 { return raw_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u); };
 #else
     intx4 stage_a[A_ITERS], stage_b[B_ITERS];
     auto load_global = [&](int k0) {
@@ -299,65 +324,89 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
 
 #if DIRECT_TO_LDS
-    // Two LDS stages.  Per K tile: read the fragments of k-steps 1.. of the current stage, start the
-    // direct-to-LDS copy of the next tile into the other stage, run the MFMAs of all but the last
-    // k-step, wait for the copy and synchronise, read the first k-step's fragments of the next tile, and
-    // run the last k-step's MFMAs underneath those reads.
-    if (ktiles > 0) copy_tile(0, k_begin);
-    wait_vmcnt0();
-    __syncthreads();
-    half8 a0[TM], b0[TN];
+    // Software pipeline over K tiles with an LDS ring of STAGES stages (tile t lives in stage t % STAGES):
+    //   * the copy of tile t+STAGES-1 is issued during k-step 0 of tile t, into the stage tile t-1 used;
+    //   * during the MFMAs of k-step s the fragments of k-step s+1 are read from LDS (two register sets);
+    //   * before the last k-step the wave waits for its own copies of tile t+1, the workgroup barrier
+    //     publishes that stage, and the last k-step's MFMAs run over the reads of tile t+1's first fragments.
+    // Every MFMA is followed by its share of the LDS reads / copy instructions and a scheduling fence, so
+    // the matrix pipe always has the next MFMA queued while the memory instructions issue in its shadow.
+    constexpr int NM = TM * TN;                    // MFMAs per k-step
+    constexpr int NR = TM + TN;                    // fragment reads per k-step
+    constexpr int NV = A_ITERS + B_ITERS;          // copy instructions per K tile
+    constexpr int RPM = (NR + NM - 1) / NM;        // reads issued behind each MFMA
+    constexpr int VPM = (NV + NM - 1) / NM;        // copies issued behind each MFMA (k-step 0 only)
+    half8 fa[2][TM], fb[2][TN];
+
+    // fragment read order: a[0], b[0..TN-1], a[1..TM-1] -- the order the MFMAs below first need them
+    auto read_frag = [&](int idx, int set, const unsigned char* sb, int step) {
+        if (idx == 0) fa[set][0] = read_a(sb, step, 0);
+        else if (idx <= TN) fb[set][idx - 1] = read_b(sb, step, idx - 1);
+        else fa[set][idx - TN] = read_a(sb, step, idx - TN);
+    };
+
     if (ktiles > 0) {
+        // prologue: tiles 0 .. STAGES-2 in flight, tile 0 complete and published
 #pragma unroll
-        for (int i = 0; i < TM; i++) a0[i] = read_a(smem, 0, i);
+        for (int t = 0; t < STAGES - 1; t++) {
+            if (t < ktiles) {
+                const int k0 = k_begin + t * BK;
+                const bool tail = (k0 + BK > p.K);
+                const intx4 ra = rsrc_a(k0), rb = rsrc_b(k0);
 #pragma unroll
-        for (int j = 0; j < TN; j++) b0[j] = read_b(smem, 0, j);
-    }
-    for (int kt = 0; kt < ktiles; kt++) {
-        const int cur = kt & 1;
-        const bool more = (kt + 1 < ktiles);
-        const unsigned char* sb = smem + cur * STAGE_BYTES;
-        half8 af[KSTEPS][TM], bf[KSTEPS][TN];
-#pragma unroll
-        for (int s = 1; s < KSTEPS; s++) {
-#pragma unroll
-            for (int i = 0; i < TM; i++) af[s][i] = read_a(sb, s, i);
-#pragma unroll
-            for (int j = 0; j < TN; j++) bf[s][j] = read_b(sb, s, j);
+                for (int idx = 0; idx < NV; idx++) copy_slot(idx, t, k0, tail, ra, rb);
+            }
         }
-        if (more) copy_tile(cur ^ 1, k_begin + (kt + 1) * BK);
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a0[i], b0[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-        for (int s = 1; s < KSTEPS - 1; s++)
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[s][i], bf[s][j], acc[i][j], 0, 0, 0);
-        // keep the instruction scheduler from hoisting the wait and barrier above the MFMAs that hide the copy
-        __builtin_amdgcn_sched_barrier(0);
-        wait_vmcnt0();
+        if (ktiles > 1 && STAGES > 2) wait_vmcnt<(STAGES - 2) * NV>(); else wait_vmcnt<0>();
         __syncthreads();
-        __builtin_amdgcn_sched_barrier(0);
-        if (more) {
-            const unsigned char* sn = smem + (cur ^ 1) * STAGE_BYTES;
 #pragma unroll
-            for (int i = 0; i < TM; i++) a0[i] = read_a(sn, 0, i);
+        for (int idx = 0; idx < NR; idx++) read_frag(idx, 0, smem, 0);
+    }
+
+    int stage_cur = 0;
+    for (int kt = 0; kt < ktiles; kt++) {
+        const unsigned char* sb = smem + stage_cur * STAGE_BYTES;
+        const int stage_nxt = (stage_cur + 1 == STAGES) ? 0 : stage_cur + 1;
+        const int stage_cpy = (stage_cur == 0) ? STAGES - 1 : stage_cur - 1;   // stage of tile kt-1 == tile kt+STAGES-1
+        const int kt_cpy = kt + STAGES - 1;
+        const bool do_copy = kt_cpy < ktiles;
+        const int k0c = k_begin + kt_cpy * BK;
+        const bool tailc = (k0c + BK > p.K);
+        // past the last tile the copy still issues, with empty descriptors: it writes zeros into a stage
+        // nobody reads again, which keeps the loop body free of branches
+        intx4 ra = rsrc_a(k0c), rb = rsrc_b(k0c);
+        if (!do_copy) { ra[2] = 0; rb[2] = 0; }
+
 #pragma unroll
-            for (int j = 0; j < TN; j++) b0[j] = read_b(sn, 0, j);
+        for (int s = 0; s < KSTEPS; s++) {
+            const int cur = s & 1, nxt = cur ^ 1;
+            if (s == KSTEPS - 1) {
+                // tile kt+1 must be complete in LDS before its first fragments are read
+                __builtin_amdgcn_sched_barrier(0);
+                if (kt + 2 < ktiles && STAGES > 2) wait_vmcnt<(STAGES - 2) * NV>(); else wait_vmcnt<0>();
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            const bool last = (s == KSTEPS - 1);
+            const unsigned char* rd_base = last ? smem + stage_nxt * STAGE_BYTES : sb;
+            const int rd_step = last ? 0 : s + 1;
+#pragma unroll
+            for (int m = 0; m < NM; m++) {
+                const int i = m / TN, j = m % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+                // (after the last tile these reads fetch an unused stage; their values are never consumed)
+#pragma unroll
+                for (int r = 0; r < RPM; r++)
+                    if (m * RPM + r < NR) read_frag(m * RPM + r, nxt, rd_base, rd_step);
+                if (s == 0) {
+#pragma unroll
+                    for (int v = 0; v < VPM; v++)
+                        if (m * VPM + v < NV) copy_slot(m * VPM + v, stage_cpy, k0c, tailc, ra, rb);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
-        if (KSTEPS > 1) {
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[KSTEPS - 1][i], bf[KSTEPS - 1][j], acc[i][j],
-                                                                       0, 0, 0);
-        }
+        stage_cur = stage_nxt;
     }
 #else
     if (ktiles > 0) {
