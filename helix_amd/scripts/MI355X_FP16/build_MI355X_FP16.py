@@ -18,7 +18,7 @@ from utils.helix_runtime import SRC_ROOT, bin_dir, compile_many
 
 root_path = os.getcwd()
 
-LDS_STAGES_LIST = [2]
+LDS_STAGES_LIST = [2, 3]
 WAVE_TILE_LIST = [32, 64, 128]
 BLOCK_SCALE_LIST = [1, 2, 4]
 BLOCK_K_LIST = [32, 64]
@@ -46,6 +46,11 @@ def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, 
     if (block_rows * chunks_per_row) % threads or (block_cols * chunks_per_row) % threads:
         return False
     if threads % chunks_per_row:
+        return False
+    # copy instructions of the later ring stages stay in flight while the wave waits for the next one:
+    # the hardware's outstanding-load counter holds 6 bits
+    copies_per_tile = (block_rows + block_cols) * chunks_per_row // threads
+    if (lds_stages - 1) * copies_per_tile > 63:
         return False
     return True
 

@@ -92,7 +92,7 @@ static_assert((BM * KCH) % NTHREADS == 0 && (BN * KCH) % NTHREADS == 0, "tile co
 #if DIRECT_TO_LDS
 static_assert(STAGES >= 2 && STAGES <= 4, "LDS ring depth must be 2..4");
 static_assert((BK / 16) % 2 == 0, "BLOCK_K must hold an even number of 16-wide MFMA k-steps");
-static_assert((STAGES - 2) * (A_ITERS + B_ITERS) <= 63, "too many copy instructions in flight for vmcnt");
+static_assert((STAGES - 1) * (A_ITERS + B_ITERS) <= 63, "too many copy instructions in flight for vmcnt");
 #else
 static_assert(STAGES == 2, "the register-staged variant implements the two-stage ring only");
 #endif
@@ -325,17 +325,19 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 
 #if DIRECT_TO_LDS
     // Software pipeline over K tiles with an LDS ring of STAGES stages (tile t lives in stage t % STAGES):
-    //   * the copy of tile t+STAGES-1 is issued during k-step 0 of tile t, into the stage tile t-1 used;
     //   * during the MFMAs of k-step s the fragments of k-step s+1 are read from LDS (two register sets);
-    //   * before the last k-step the wave waits for its own copies of tile t+1, the workgroup barrier
-    //     publishes that stage, and the last k-step's MFMAs run over the reads of tile t+1's first fragments.
+    //   * before the last k-step of tile t the wave waits for its own copies of tile t+1 and the workgroup
+    //     barrier publishes that stage; at that point tile t's stage has been read completely (its last
+    //     fragments sit in registers), so the copy of tile t+STAGES is issued into it during the last
+    //     k-step, next to the reads of tile t+1's first fragments.  A copy therefore has a whole K tile
+    //     (STAGES-1 of them for deeper rings) to land before anyone waits for it.
     // Every MFMA is followed by its share of the LDS reads / copy instructions and a scheduling fence, so
     // the matrix pipe always has the next MFMA queued while the memory instructions issue in its shadow.
     constexpr int NM = TM * TN;                    // MFMAs per k-step
     constexpr int NR = TM + TN;                    // fragment reads per k-step
     constexpr int NV = A_ITERS + B_ITERS;          // copy instructions per K tile
     constexpr int RPM = (NR + NM - 1) / NM;        // reads issued behind each MFMA
-    constexpr int VPM = (NV + NM - 1) / NM;        // copies issued behind each MFMA (k-step 0 only)
+    constexpr int VPM = (NV + NM - 1) / NM;        // copies issued behind each MFMA (last k-step only)
     half8 fa[2][TM], fb[2][TN];
 
     // fragment read order: a[0], b[0..TN-1], a[1..TM-1] -- the order the MFMAs below first need them
@@ -346,9 +348,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     };
 
     if (ktiles > 0) {
-        // prologue: tiles 0 .. STAGES-2 in flight, tile 0 complete and published
+        // prologue: tiles 0 .. STAGES-1 in flight, tile 0 complete and published
 #pragma unroll
-        for (int t = 0; t < STAGES - 1; t++) {
+        for (int t = 0; t < STAGES; t++) {
             if (t < ktiles) {
                 const int k0 = k_begin + t * BK;
                 const bool tail = (k0 + BK > p.K);
@@ -357,7 +359,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
                 for (int idx = 0; idx < NV; idx++) copy_slot(idx, t, k0, tail, ra, rb);
             }
         }
-        if (ktiles > 1 && STAGES > 2) wait_vmcnt<(STAGES - 2) * NV>(); else wait_vmcnt<0>();
+        // the copies complete in issue order: allow the later tiles' copies to stay in flight
+        if (ktiles >= STAGES) wait_vmcnt<(STAGES - 1) * NV>(); else wait_vmcnt<0>();
         __syncthreads();
 #pragma unroll
         for (int idx = 0; idx < NR; idx++) read_frag(idx, 0, smem, 0);
@@ -367,27 +370,26 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     for (int kt = 0; kt < ktiles; kt++) {
         const unsigned char* sb = smem + stage_cur * STAGE_BYTES;
         const int stage_nxt = (stage_cur + 1 == STAGES) ? 0 : stage_cur + 1;
-        const int stage_cpy = (stage_cur == 0) ? STAGES - 1 : stage_cur - 1;   // stage of tile kt-1 == tile kt+STAGES-1
-        const int kt_cpy = kt + STAGES - 1;
-        const bool do_copy = kt_cpy < ktiles;
+        const int kt_cpy = kt + STAGES;            // tile copied into stage_cur once tile kt has been read
         const int k0c = k_begin + kt_cpy * BK;
         const bool tailc = (k0c + BK > p.K);
         // past the last tile the copy still issues, with empty descriptors: it writes zeros into a stage
         // nobody reads again, which keeps the loop body free of branches
         intx4 ra = rsrc_a(k0c), rb = rsrc_b(k0c);
-        if (!do_copy) { ra[2] = 0; rb[2] = 0; }
+        if (kt_cpy >= ktiles) { ra[2] = 0; rb[2] = 0; }
 
 #pragma unroll
         for (int s = 0; s < KSTEPS; s++) {
             const int cur = s & 1, nxt = cur ^ 1;
-            if (s == KSTEPS - 1) {
-                // tile kt+1 must be complete in LDS before its first fragments are read
+            const bool last = (s == KSTEPS - 1);
+            if (last) {
+                // tile kt+1 must be complete in LDS before its first fragments are read; the copies of
+                // tiles kt+2 .. kt+STAGES-1 (issued later) may stay in flight
                 __builtin_amdgcn_sched_barrier(0);
-                if (kt + 2 < ktiles && STAGES > 2) wait_vmcnt<(STAGES - 2) * NV>(); else wait_vmcnt<0>();
+                if (STAGES > 2 && kt + STAGES - 1 < ktiles) wait_vmcnt<(STAGES - 2) * NV>(); else wait_vmcnt<0>();
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            const bool last = (s == KSTEPS - 1);
             const unsigned char* rd_base = last ? smem + stage_nxt * STAGE_BYTES : sb;
             const int rd_step = last ? 0 : s + 1;
 #pragma unroll
@@ -398,10 +400,10 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 #pragma unroll
                 for (int r = 0; r < RPM; r++)
                     if (m * RPM + r < NR) read_frag(m * RPM + r, nxt, rd_base, rd_step);
-                if (s == 0) {
+                if (last) {
 #pragma unroll
                     for (int v = 0; v < VPM; v++)
-                        if (m * VPM + v < NV) copy_slot(m * VPM + v, stage_cpy, k0c, tailc, ra, rb);
+                        if (m * VPM + v < NV) copy_slot(m * VPM + v, stage_cur, k0c, tailc, ra, rb);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }

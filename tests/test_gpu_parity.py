@@ -76,7 +76,8 @@ def run_sgemm_f32(lib, A, B):
 
 
 FP16_CONFIGS = [(2, 256, 256, 128, 128, 64), (2, 256, 256, 64, 128, 64), (2, 128, 128, 64, 64, 32), (2, 64, 64, 32, 32, 64),
-                (2, 32, 32, 32, 32, 32), (2, 256, 64, 64, 32, 64), (2, 64, 256, 32, 128, 32), (2, 128, 256, 128, 64, 64)]
+                (2, 32, 32, 32, 32, 32), (2, 256, 64, 64, 32, 64), (2, 64, 256, 32, 128, 32), (2, 128, 256, 128, 64, 64),
+                (3, 128, 128, 64, 64, 64), (3, 256, 256, 128, 128, 32), (3, 64, 64, 32, 32, 32), (3, 32, 128, 32, 64, 64)]
 
 
 # ---------------------------------------------------------------------------------------------
@@ -265,7 +266,7 @@ CONV_GEOMS = [(2, 14, 14, 16, 24, 3, 3, 1, 1), (2, 15, 13, 8, 8, 3, 3, 2, 1), (3
 
 
 @pytest.mark.parametrize("cfg", [(2, 128, 128, 64, 64, 64), (2, 64, 64, 32, 32, 32), (2, 256, 64, 64, 32, 64),
-                                 (2, 128, 64, 64, 32, 32)])
+                                 (2, 128, 64, 64, 32, 32), (3, 128, 128, 64, 64, 32), (3, 64, 128, 32, 64, 64)])
 def test_conv_f16_vs_oracle(cfg):
     lib = load(b16.kernel_library("gemm", *cfg))
     for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS:

@@ -22,6 +22,7 @@ from MI355X_FP32 import profile_MI355X_FP32 as p32
 from MI355X_FP32 import MI355X_FP32_gemm as g32
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+N_FP16_CONFIGS = 220   # 112 two-stage + 108 three-stage points of the FP16 tile / wave / BLOCK_K / ring-depth space
 
 
 # ---- enumeration ----------------------------------------------------------------------------------
@@ -38,15 +39,16 @@ def test_fp16_reference_validity_rules():
 
 def test_fp16_template_space():
     cfgs = list(b16.iter_configs())
-    assert len(cfgs) == 112 and len(set(cfgs)) == 112
+    assert len(cfgs) == N_FP16_CONFIGS and len(set(cfgs)) == N_FP16_CONFIGS
     for (st, br, bc, wr, wc, bk) in cfgs:
         assert br % wr == 0 and bc % wc == 0 and br <= 256 and bc <= 256
         assert st * (br + bc) * bk * 2 <= 160 * 1024
         threads = 64 * (br // wr) * (bc // wc)
         assert threads <= 512 and (br * bk // 8) % threads == 0 and (bc * bk // 8) % threads == 0
+        assert (st - 1) * ((br + bc) * (bk // 8) // threads) <= 63
     assert (2, 256, 256, 128, 128, 64) in cfgs
     keys = p16.all_keys()
-    assert len(keys) == 2 * 112 + 6
+    assert len(keys) == 2 * N_FP16_CONFIGS + 6
     assert all(len(k) == 7 for k in keys)
     assert sum(1 for k in keys if k[0] == 0) == 6   # GEMV rows are tagged by a zero first field
 
