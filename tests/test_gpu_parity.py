@@ -230,7 +230,9 @@ def test_gemv_f16_baseline_shapes_sampled():
             Wt = np.ascontiguousarray(W.T)
             dx, dW = dev(x), dev(Wt)
             dy = torch.empty((M, N), dtype=torch.float16, device="cuda:0")
-            lib.gemm(dx.data_ptr(), dW.data_ptr(), dy.data_ptr(), M, N, K, K, K, N)
+            wsb = lib.workspace_bytes(M, N, K)   # wide activation tiles partition K and need FP32 scratch
+            ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda:0")
+            lib.gemm(dx.data_ptr(), dW.data_ptr(), dy.data_ptr(), M, N, K, K, K, N, ws.data_ptr(), wsb)
             torch.cuda.synchronize()
             y = dy.cpu().numpy()
             cols = np.concatenate([rng.integers(0, N, 200), [0, N - 1]])
