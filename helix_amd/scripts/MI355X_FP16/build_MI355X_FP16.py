@@ -18,7 +18,8 @@ from utils.helix_runtime import SRC_ROOT, bin_dir, compile_many
 
 root_path = os.getcwd()
 
-LDS_STAGES_LIST = [2, 3]
+LDS_STAGES_LIST = [2, 3, 4]
+SPLITK_STAGES_LIST = [2]    # split-K variants are built for the two-stage ring only (tiny M x N problems)
 WAVE_TILE_LIST = [32, 64, 128]
 BLOCK_SCALE_LIST = [1, 2, 4]
 BLOCK_K_LIST = [32, 64]
@@ -122,7 +123,8 @@ def build_jobs():
     jobs = []
     for cfg in iter_configs():
         jobs.append(compile_job("gemm", *cfg))
-        jobs.append(compile_job("gemm_splitK", *cfg))
+        if cfg[0] in SPLITK_STAGES_LIST:
+            jobs.append(compile_job("gemm_splitK", *cfg))
     jobs.append(compile_job("gemv"))
     jobs.append(compile_job("gemv_splitK"))
     return jobs

@@ -9,7 +9,7 @@ from tqdm import tqdm
 
 from utils.helix_runtime import write_prof_dict
 from MI355X_FP16.build_MI355X_FP16 import (LDS_STAGES_LIST, WAVE_TILE_LIST, BLOCK_SCALE_LIST, BLOCK_K_LIST,
-                                           is_valid_config)
+                                           is_valid_config, SPLITK_STAGES_LIST)
 from MI355X_FP16.profile_MI355X_FP16 import time_config, GEMV_KEYS, GEMV_SPLITK_KEYS
 
 root_path = os.getcwd()
@@ -29,6 +29,8 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
                     for BLOCK_K in BLOCK_K_LIST:
                         for splitK in (0, 1):
                             pbar.update(1)
+                            if splitK == 1 and LDS_STAGES not in SPLITK_STAGES_LIST:
+                                continue
                             if not is_valid_config(1, 1, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K, LDS_STAGES):
                                 continue
                             cost = time_config((LDS_STAGES, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K))

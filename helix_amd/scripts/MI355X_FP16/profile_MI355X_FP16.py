@@ -13,7 +13,7 @@ from tqdm import tqdm
 
 from utils.helix_runtime import load, write_prof_dict
 from utils.roofline import NUM_CU
-from MI355X_FP16.build_MI355X_FP16 import iter_configs, library_for_key
+from MI355X_FP16.build_MI355X_FP16 import iter_configs, library_for_key, SPLITK_STAGES_LIST
 
 root_path = os.getcwd()
 
@@ -55,7 +55,8 @@ def all_keys():
     keys = []
     for (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in iter_configs():
         keys.append((LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 0, BLOCK_K))
-        keys.append((LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 1, BLOCK_K))
+        if LDS_STAGES in SPLITK_STAGES_LIST:
+            keys.append((LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 1, BLOCK_K))
     keys.extend(GEMV_KEYS)
     keys.extend(GEMV_SPLITK_KEYS)
     return keys

@@ -69,6 +69,8 @@ namespace {
 typedef _Float16 half_t;
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
 
 constexpr int BM = BLOCK_ROWS, BN = BLOCK_COLS, WM = WAVE_ROWS, WN = WAVE_COLS, BK = BLOCK_K;
@@ -82,7 +84,11 @@ constexpr int A_ITERS = BM * KCH / NTHREADS, B_ITERS = BN * KCH / NTHREADS;
 constexpr int ROWS_PER_ITER = NTHREADS / KCH;
 constexpr int A_STAGE_BYTES = BM * ROW_BYTES, B_STAGE_BYTES = BN * ROW_BYTES;
 constexpr int STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
-constexpr int LDS_BYTES = STAGES * STAGE_BYTES;
+constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+// epilogue staging: one 32 x WAVE_COLS strip of halves per wave, rows padded by 16 bytes
+constexpr int STRIP_LD = WN * 2 + 16;
+constexpr int STRIP_BYTES = 32 * STRIP_LD;
+constexpr int LDS_BYTES = RING_BYTES > NWAVES * STRIP_BYTES ? RING_BYTES : NWAVES * STRIP_BYTES;
 
 static_assert(BM % WM == 0 && BN % WN == 0, "block tile must be a multiple of the wave tile");
 static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is built from 32x32 MFMA tiles");
@@ -153,9 +159,13 @@ __device__ __forceinline__ intx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) 
 
 // The tile parameters appear as (otherwise unused) template arguments so that every configuration's
 // kernel has its own symbol name and a profiler lists configurations separately.
-template <bool CONV, int T_STAGES = STAGES, int T_BM = BM, int T_BN = BN, int T_WM = WM, int T_WN = WN, int T_BK = BK,
+// MODE: 0 = GEMM; 1 = convolution, general gather (tap and channel of every 16-byte chunk computed per K
+// tile); 2 = convolution with IC a multiple of BLOCK_K and at most 32 filter taps: a K tile then lies inside
+// one filter tap, so the tap offset is one scalar per tile and each copy slot only tests its tap-validity bit.
+template <int MODE, int T_STAGES = STAGES, int T_BM = BM, int T_BN = BN, int T_WM = WM, int T_WN = WN, int T_BK = BK,
           int T_SPLITK = SPLITK>
 __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p) {
+    constexpr bool CONV = (MODE != 0);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const int tid = threadIdx.x;
@@ -216,6 +226,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     unsigned bytesA = 0;
     int voff_a[A_ITERS];
     int cv_img[A_ITERS], cv_ih[A_ITERS], cv_iw[A_ITERS];  // CONV: image base offset, top-left tap coords
+    int cv_base[A_ITERS];                                 // MODE 2: byte offset of the row's top-left tap + chunk
+    unsigned cv_taps[A_ITERS];                            // MODE 2: bit t set = filter tap t reads inside the image
     if (!CONV) {
         const int rows_a = (p.M - m0) < BM ? (p.M - m0) : BM;
         baseA = p.A + (size_t)m0 * p.lda;
@@ -235,14 +247,38 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             cv_img[i] = (m < p.g.M) ? b * p.g.H * p.g.W : -1;
             cv_ih[i] = oh * p.g.stride - p.g.pad;
             cv_iw[i] = ow * p.g.stride - p.g.pad;
+            if (MODE == 2) {
+                cv_base[i] = ((cv_img[i] + cv_ih[i] * p.g.W + cv_iw[i]) * p.g.IC + gch_a[i] * 8) * 2;
+                unsigned taps = 0;
+                const int ntaps = p.K / p.g.IC;
+                for (int t = 0; t < ntaps; t++) {
+                    const int ih = cv_ih[i] + t / p.g.kW, iw = cv_iw[i] + t % p.g.kW;
+                    if (cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W) taps |= 1u << t;
+                }
+                cv_taps[i] = taps;
+            }
         }
     }
 
+    // MODE 2: scalar state of the K tile at k0: byte offset of its filter tap and channel block, and its tap bit
+    struct ConvTile { int soff; unsigned tapbit; };
+    auto conv_tile = [&](int k0) -> ConvTile {
+        ConvTile ct{0, 0u};
+        if (MODE == 2 && k0 < p.K) {
+            const int tap = k0 / p.g.IC, c0 = k0 % p.g.IC;
+            ct.soff = (((tap / p.g.kW) * p.g.W + tap % p.g.kW) * p.g.IC + c0) * 2;
+            ct.tapbit = 1u << tap;
+        }
+        return ct;
+    };
+
     // Byte offset (relative to the operand's buffer descriptor) of copy slot i for the K tile at k0, or
     // OOB_OFFSET when the slot must read zeros (beyond K, conv padding, rows beyond M).
-    auto a_offset = [&](int i, int k0, bool tail) -> int {
+    auto a_offset = [&](int i, int k0, bool tail, ConvTile ct) -> int {
         if (!CONV) {
             return (tail && k0 + gch_a[i] * 8 >= p.K) ? OOB_OFFSET : voff_a[i];
+        } else if (MODE == 2) {
+            return (cv_taps[i] & ct.tapbit) ? cv_base[i] + ct.soff : OOB_OFFSET;
         } else {
             const int k = k0 + gch_a[i] * 8;  // k = (kh*kW + kw)*IC + c, 8 consecutive c per chunk
             const int c = k % p.g.IC;
@@ -266,9 +302,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     const unsigned lds_base = (unsigned)(uintptr_t)(lds_ptr_t)smem;
     const unsigned lds_wave = lds_base + (unsigned)wave * 1024u;
     // copy slot `idx` (A slots first, then B slots) of the K tile at k0 into LDS stage `stage`
-    auto copy_slot = [&](int idx, int stage, int k0, bool tail, intx4 ra, intx4 rb) {
+    auto copy_slot = [&](int idx, int stage, int k0, bool tail, intx4 ra, intx4 rb, ConvTile ct) {
         if (idx < A_ITERS) {
-            const int off = a_offset(idx, k0, tail);
+            const int off = a_offset(idx, k0, tail, ct);
             dma16(ra, lds_wave + (unsigned)(stage * STAGE_BYTES + idx * NTHREADS * 16), off);
         } else {
             const int i = idx - A_ITERS;
@@ -288,8 +324,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         __amdgpu_buffer_rsrc_t ra = CONV ? make_rsrc(baseA, bytesA) : make_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
 #pragma unroll
         for (int i = 0; i < B_ITERS; i++) stage_b[i] = buf_load16(rb, b_offset(i, k0, tail));
+        const ConvTile ct = conv_tile(k0);
 #pragma unroll
-        for (int i = 0; i < A_ITERS; i++) stage_a[i] = buf_load16(ra, a_offset(i, k0, tail));
+        for (int i = 0; i < A_ITERS; i++) stage_a[i] = buf_load16(ra, a_offset(i, k0, tail, ct));
     };
     auto store_lds = [&](int stage) {
         unsigned char* base = smem + stage * STAGE_BYTES + tid * 16;
@@ -355,8 +392,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
                 const int k0 = k_begin + t * BK;
                 const bool tail = (k0 + BK > p.K);
                 const intx4 ra = rsrc_a(k0), rb = rsrc_b(k0);
+                const ConvTile ct = conv_tile(k0);
 #pragma unroll
-                for (int idx = 0; idx < NV; idx++) copy_slot(idx, t, k0, tail, ra, rb);
+                for (int idx = 0; idx < NV; idx++) copy_slot(idx, t, k0, tail, ra, rb, ct);
             }
         }
         // the copies complete in issue order: allow the later tiles' copies to stay in flight
@@ -377,6 +415,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         // nobody reads again, which keeps the loop body free of branches
         intx4 ra = rsrc_a(k0c), rb = rsrc_b(k0c);
         if (kt_cpy >= ktiles) { ra[2] = 0; rb[2] = 0; }
+        const ConvTile ctc = conv_tile(k0c);
 
 #pragma unroll
         for (int s = 0; s < KSTEPS; s++) {
@@ -395,7 +434,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 #pragma unroll
             for (int m = 0; m < NM; m++) {
                 const int i = m / TN, j = m % TN;
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[cur][i], fb[cur][j], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
                 // (after the last tile these reads fetch an unused stage; their values are never consumed)
 #pragma unroll
                 for (int r = 0; r < RPM; r++)
@@ -403,7 +442,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
                 if (last) {
 #pragma unroll
                     for (int v = 0; v < VPM; v++)
-                        if (m * VPM + v < NV) copy_slot(m * VPM + v, stage_cur, k0c, tailc, ra, rb);
+                        if (m * VPM + v < NV) copy_slot(m * VPM + v, stage_cur, k0c, tailc, ra, rb, ctc);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -434,7 +473,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
         }
 
         if (more) store_lds(cur ^ 1);
@@ -442,23 +481,79 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     }
 #endif
 
-    // ---- epilogue: lane l holds column (l % 32); rows 8*(v/4) + 4*(l/32) + (v%4), v = 0..15 -------
-    const int col_l = lane & 31, row_l = (lane >> 5) * 4;
+    // ---- epilogue ---------------------------------------------------------------------------------
+    // The MFMAs were issued with the B fragment as the first operand, so accumulator tile (i, j) holds the
+    // transposed 32x32 block: lane l owns tile row m = l % 32 and, in registers 4g..4g+3, the four
+    // consecutive tile columns n = 8g + 4*(l/32) + {0,1,2,3}.
+    const int m_l = lane & 31, n_l = (lane >> 5) * 4;
+    if (SPLITK > 1) {
+        // FP32 partial sums: four consecutive columns per lane, one 16-byte store where that is aligned
+        const bool vec_ok = (p.N % 4 == 0);
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+        for (int i = 0; i < TM; i++) {
+            const int row = m0 + wave_m * WM + i * 32 + m_l;
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int col = n0 + wave_n * WN + j * 32 + col_l;
+            for (int j = 0; j < TN; j++) {
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const int row = m0 + wave_m * WM + i * 32 + (v / 4) * 8 + row_l + (v % 4);
-                if (row < p.M && col < p.N) {
-                    if (SPLITK > 1)
-                        p.ws[((size_t)blockIdx.y * p.M + row) * p.N + col] = acc[i][j][v];
-                    else
-                        p.C[(size_t)row * p.ldc + col] = (half_t)acc[i][j][v];
+                for (int g = 0; g < 4; g++) {
+                    const int col = n0 + wave_n * WN + j * 32 + g * 8 + n_l;
+                    if (row < p.M) {
+                        float* dst = p.ws + ((size_t)blockIdx.y * p.M + row) * p.N + col;
+                        if (vec_ok && col + 4 <= p.N) {
+                            floatx4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                            *(floatx4*)dst = v;
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                if (col + e < p.N) dst[e] = acc[i][j][4 * g + e];
+                        }
+                    }
                 }
             }
+        }
+    } else {
+        // FP16 result through LDS: each wave rounds a 32 x WAVE_COLS strip into its private LDS region
+        // (8-byte writes), reads it back row-contiguous and stores 16 bytes per lane, so a store
+        // instruction covers whole 2*WAVE_COLS-byte row segments.
+#if DIRECT_TO_LDS
+        wait_vmcnt<0>();   // the (empty) copies issued behind the last tiles still write zeros into the ring
+#endif
+        __syncthreads();   // every wave is done reading the ring; the strips reuse its memory
+        unsigned char* strip = smem + wave * STRIP_BYTES;
+        const bool vec_ok = (p.ldc % 8 == 0) && (((uintptr_t)p.C & 15) == 0);
+        constexpr int CPR = WN / 8;                    // 16-byte chunks per strip row
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    half4 h = {(half_t)acc[i][j][4 * g], (half_t)acc[i][j][4 * g + 1], (half_t)acc[i][j][4 * g + 2],
+                               (half_t)acc[i][j][4 * g + 3]};
+                    *(half4*)(strip + m_l * STRIP_LD + (j * 32 + g * 8 + n_l) * 2) = h;
+                }
+            }
+            __builtin_amdgcn_wave_barrier();   // same-wave LDS traffic stays in program order
+#pragma unroll
+            for (int t = 0; t < (32 * CPR) / 64; t++) {
+                const int idx = t * 64 + lane;
+                const int r = idx / CPR, ch = idx % CPR;
+                const intx4 v = *(const intx4*)(strip + r * STRIP_LD + ch * 16);
+                const int row = m0 + wave_m * WM + i * 32 + r;
+                const int col = n0 + wave_n * WN + ch * 8;
+                if (row < p.M && col < p.N) {
+                    half_t* dst = p.C + (size_t)row * p.ldc + col;
+                    if (vec_ok && col + 8 <= p.N) {
+                        *(intx4*)dst = v;
+                    } else {
+                        const half8 hv = __builtin_bit_cast(half8, v);
+#pragma unroll
+                        for (int e = 0; e < 8; e++)
+                            if (col + e < p.N) dst[e] = hv[e];
+                    }
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
         }
     }
 }
@@ -514,25 +609,25 @@ inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce
     *lda = K; *ldb = K; *ldc = N;
 }
 
-template <bool CONV>
+template <int MODE>
 inline int set_lds_attr() {
-    static int rc = (int)hipFuncSetAttribute((const void*)helix_gemm_f16_kernel<CONV>,
+    static int rc = (int)hipFuncSetAttribute((const void*)helix_gemm_f16_kernel<MODE>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     return rc;
 }
 
-template <bool CONV>
+template <int MODE>
 inline int launch(const Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
     if (SPLITK > 1) {
         const size_t need = workspace_bytes(p.M, p.N, p.K);
         if (!ws || ws_bytes < need) return HELIX_ERR_WORKSPACE;
     }
-    int rc = set_lds_attr<CONV>();
+    int rc = set_lds_attr<MODE>();
     if (rc) return rc;
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
     dim3 grid((unsigned)ntiles, SPLITK, 1), block(NTHREADS, 1, 1);
-    hipLaunchKernelGGL(helix_gemm_f16_kernel<CONV>, grid, block, LDS_BYTES, s, p);
+    hipLaunchKernelGGL(helix_gemm_f16_kernel<MODE>, grid, block, LDS_BYTES, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     if (SPLITK > 1) {
@@ -559,7 +654,7 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     p.A = (const half_t*)A; p.B = (const half_t*)B; p.C = (half_t*)C; p.ws = (float*)ws;
     p.M = M; p.N = N; p.K = K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
     p.tiles_m = (M + BM - 1) / BM; p.tiles_n = (N + BN - 1) / BN;
-    return launch<false>(p, ws, ws_bytes, s);
+    return launch<0>(p, ws, ws_bytes, s);
 }
 
 inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
@@ -577,7 +672,9 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
     p.tiles_m = (int)((M + BM - 1) / BM); p.tiles_n = (OC + BN - 1) / BN;
     p.a_bytes = (unsigned)xbytes;
     p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M};
-    return launch<true>(p, ws, ws_bytes, s);
+    // a K tile inside one filter tap (and a tap mask that fits 32 bits) takes the scalar-tap gather
+    if (IC % BK == 0 && kH * kW <= 32) return launch<2>(p, ws, ws_bytes, s);
+    return launch<1>(p, ws, ws_bytes, s);
 }
 
 }  // namespace tpl

@@ -22,7 +22,8 @@ from MI355X_FP32 import profile_MI355X_FP32 as p32
 from MI355X_FP32 import MI355X_FP32_gemm as g32
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-N_FP16_CONFIGS = 220   # 112 two-stage + 108 three-stage points of the FP16 tile / wave / BLOCK_K / ring-depth space
+N_FP16_CONFIGS = 316   # 112 two-stage + 108 three-stage + 96 four-stage points of the FP16 template space
+N_FP16_SPLITK = 112    # split-K variants exist for the two-stage ring only
 
 
 # ---- enumeration ----------------------------------------------------------------------------------
@@ -48,7 +49,7 @@ def test_fp16_template_space():
         assert (st - 1) * ((br + bc) * (bk // 8) // threads) <= 63
     assert (2, 256, 256, 128, 128, 64) in cfgs
     keys = p16.all_keys()
-    assert len(keys) == 2 * N_FP16_CONFIGS + 6
+    assert len(keys) == N_FP16_CONFIGS + N_FP16_SPLITK + 6
     assert all(len(k) == 7 for k in keys)
     assert sum(1 for k in keys if k[0] == 0) == 6   # GEMV rows are tagged by a zero first field
 
