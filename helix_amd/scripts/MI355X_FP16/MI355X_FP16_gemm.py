@@ -9,13 +9,26 @@ import os
 
 from utils.helix_runtime import load
 from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
-from MI355X_FP16.build_MI355X_FP16 import library_for_key
+from MI355X_FP16.build_MI355X_FP16 import library_for_key, SPLITK_MAX
 from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K
 
 root_path = os.getcwd()
 
 HBM_SUSTAINED_FRACTION = 0.6  # share of the datasheet HBM rate a streaming kernel sustains
-GEMV_LAUNCH_FLOOR_S = 3e-6   # a kernel launch on an idle queue; keeps tiny problems from looking free
+GEMV_LAUNCH_FLOOR_S = 3e-6
+SPLITK_REDUCE_LAUNCH_S = 4e-6  # the reduction kernel's launch, beyond what the profiled value already holds   # a kernel launch on an idle queue; keeps tiny problems from looking free
+
+
+def split_factor(k, M, N, K):
+    """K partitions a split-K library uses for this problem (same rule as the library's host side):
+    enough to give each of the 256 compute units a workgroup, between 2 and SPLITK_MAX, and at least two
+    K tiles per partition.  The reference's split is always 2 (`* (k[5] + 1)`, Ampere_FP16_gemm.py:424)."""
+    if k[5] == 0 or k[0] == 0:
+        return 1
+    tiles = math.ceil(M / k[1]) * math.ceil(N / k[2])
+    ktiles = math.ceil(K / k[6])
+    s = min(NUM_CU // max(tiles, 1), SPLITK_MAX, ktiles // 2)
+    return max(s, 2)
 
 
 def config_cost(k, v, M, N, K):
@@ -30,13 +43,20 @@ def config_cost(k, v, M, N, K):
         small, big = (M, N) if M <= N else (N, M)
         num_block = math.ceil(small / k[1]) * math.ceil(big / k[2])
         return max(num_block / NUM_CU * v * max(K, 512) / PROFILE_K, GEMV_LAUNCH_FLOOR_S)
-    num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * (k[5] + 1)
+    splits = split_factor(k, M, N, K)
+    num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * splits
     w = math.ceil(num_block / NUM_CU)
     k_scale = max(K, 64) / PROFILE_K
     if k[5] == 1:
-        k_scale = k_scale / 2 + 64 / PROFILE_K
+        # the profiled value is two rounds of half-K partitions, i.e. about one full-K round; a round of
+        # this problem walks K / splits
+        k_scale = k_scale / splits + 64 / PROFILE_K
+    cost = w * v * k_scale
+    if k[5] == 1:
+        # the FP32 partials are written and read back by a second kernel
+        cost += SPLITK_REDUCE_LAUNCH_S + (splits + 1) * M * N * 4 / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S)
     # a tile round cannot beat streaming every operand once from HBM at the sustained rate
-    return max(w * v * k_scale, gemm_bytes(M, N, K, 2) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
+    return max(cost, gemm_bytes(M, N, K, 2) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
 
 
 def cost_model(prof_dict, M, N, K):

@@ -19,6 +19,7 @@ from utils.helix_runtime import SRC_ROOT, bin_dir, compile_many
 root_path = os.getcwd()
 
 LDS_STAGES_LIST = [2, 3, 4]
+SPLITK_MAX = 8              # a split-K library partitions K 2 .. 8 ways, chosen per problem
 SPLITK_STAGES_LIST = [2]    # split-K variants are built for the two-stage ring only (tiny M x N problems)
 WAVE_TILE_LIST = [32, 64, 128]
 BLOCK_SCALE_LIST = [1, 2, 4]
@@ -98,7 +99,7 @@ def compile_job(kernel_name, lds_stages=None, block_rows=None, block_cols=None, 
     src_name = kernel_name
     if kernel_name == "gemm_splitK":
         src_name = "gemm"
-        defines["SPLIT_K"] = 2
+        defines["SPLIT_K"] = SPLITK_MAX
     elif kernel_name == "gemv_splitK":
         src_name = "gemv"
         defines["SPLIT_K"] = 4

@@ -14,7 +14,9 @@
 //   WAVE_ROWS  x WAVE_COLS    tile of C owned by one wave64 (reference WARP_ROWS / WARP_COLS)
 //   BLOCK_K                   K extent of one LDS stage
 //   LDS_STAGES                LDS ring depth                (reference K_STAGE)
-//   SPLIT_K                   K partitions (FP32 workspace + reduction kernel when > 1)
+//   SPLIT_K                   1: each workgroup walks all of K.  > 1: K is partitioned over blockIdx.y into
+//                             2 .. SPLIT_K ranges, as many as it takes to give every compute unit a
+//                             workgroup (FP32 workspace + fixed-order reduction kernel)
 //
 // Kernel structure
 //   * one wave64 computes (WAVE_ROWS/32) x (WAVE_COLS/32) v_mfma_f32_32x32x16_f16 tiles; per 16-wide
@@ -72,6 +74,7 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef int intx2 __attribute__((ext_vector_type(2)));
 
 constexpr int BM = BLOCK_ROWS, BN = BLOCK_COLS, WM = WAVE_ROWS, WN = WAVE_COLS, BK = BLOCK_K;
 constexpr int STAGES = LDS_STAGES, SPLITK = SPLIT_K;
@@ -113,7 +116,8 @@ struct Params {
     const half_t* A;   // GEMM: M x K (lda).  CONV: x, NHWC
     const half_t* B;   // N x K (ldb).        CONV: w, [OC][kH][kW][IC]
     half_t* C;         // M x N (ldc)
-    float* ws;         // SPLIT_K > 1: [SPLIT_K][M][N] FP32 partial sums
+    float* ws;         // SPLIT_K > 1: [splits][M][N] FP32 partial sums
+    int splits;        // K partitions of this launch (1 when SPLIT_K == 1)
     int M, N, K, lda, ldb, ldc;
     int tiles_m, tiles_n;
     unsigned a_bytes;  // CONV: size of x in bytes (bounds for the gather)
@@ -194,7 +198,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     int k_begin = 0, k_end = p.K;
     if (SPLITK > 1) {
         const int ktiles = (p.K + BK - 1) / BK;
-        const int per = (ktiles + SPLITK - 1) / SPLITK;
+        const int per = (ktiles + p.splits - 1) / p.splits;
         k_begin = (int)blockIdx.y * per * BK;
         k_end = k_begin + per * BK;
         if (k_end > p.K) k_end = p.K;
@@ -520,7 +524,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 #endif
         __syncthreads();   // every wave is done reading the ring; the strips reuse its memory
         unsigned char* strip = smem + wave * STRIP_BYTES;
-        const bool vec_ok = (p.ldc % 8 == 0) && (((uintptr_t)p.C & 15) == 0);
+        // widest store the row stride and base address allow: 8, 4, 2 or 1 halves at a time
+        const int valign = (int)(((uintptr_t)p.C >> 1) | (unsigned)p.ldc) & 7;
+        const int vec = (valign == 0) ? 8 : (valign & 3) == 0 ? 4 : (valign & 1) == 0 ? 2 : 1;
         constexpr int CPR = WN / 8;                    // 16-byte chunks per strip row
 #pragma unroll
         for (int i = 0; i < TM; i++) {
@@ -543,8 +549,14 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
                 const int col = n0 + wave_n * WN + ch * 8;
                 if (row < p.M && col < p.N) {
                     half_t* dst = p.C + (size_t)row * p.ldc + col;
-                    if (vec_ok && col + 8 <= p.N) {
+                    if (vec == 8 && col + 8 <= p.N) {
                         *(intx4*)dst = v;
+                    } else if (vec == 4 && col + 8 <= p.N) {
+                        ((intx2*)dst)[0] = intx2{v[0], v[1]};
+                        ((intx2*)dst)[1] = intx2{v[2], v[3]};
+                    } else if (vec == 2 && col + 8 <= p.N) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) ((int*)dst)[e] = v[e];
                     } else {
                         const half8 hv = __builtin_bit_cast(half8, v);
 #pragma unroll
@@ -599,9 +611,22 @@ inline const char* info_json() {
     return buf;
 }
 
+// K partitions for an M x N x K problem: enough to hand every one of the 256 compute units a workgroup,
+// at least 2 (the reference's split-K is always 2-way, gemm_splitK.cu:124-129), at most SPLIT_K, and
+// never so many that a partition has fewer than two K tiles.
+inline int split_factor(long long M, long long N, long long K) {
+    if (SPLITK <= 1) return 1;
+    const long long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    const long long ktiles = (K + BK - 1) / BK;
+    long long s = 256 / (tiles > 0 ? tiles : 1);
+    if (s > SPLITK) s = SPLITK;
+    if (s > ktiles / 2) s = ktiles / 2;
+    if (s < 2) s = 2;
+    return (int)s;
+}
+
 inline size_t workspace_bytes(int M, int N, int K) {
-    (void)K;
-    return SPLITK > 1 ? (size_t)SPLITK * (size_t)M * (size_t)N * sizeof(float) : 0;
+    return SPLITK > 1 ? (size_t)split_factor(M, N, K) * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
 inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce, int* lda, int* ldb, int* ldc) {
@@ -626,7 +651,7 @@ inline int launch(const Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
     if (rc) return rc;
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
-    dim3 grid((unsigned)ntiles, SPLITK, 1), block(NTHREADS, 1, 1);
+    dim3 grid((unsigned)ntiles, (unsigned)p.splits, 1), block(NTHREADS, 1, 1);
     hipLaunchKernelGGL(helix_gemm_f16_kernel<MODE>, grid, block, LDS_BYTES, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
@@ -635,7 +660,7 @@ inline int launch(const Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
         int blocks = (int)((total + 255) / 256);
         if (blocks > 8192) blocks = 8192;
         hipLaunchKernelGGL(helix_splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, (const float*)ws, p.C, p.M,
-                           p.N, p.ldc, SPLITK);
+                           p.N, p.ldc, p.splits);
         e = hipGetLastError();
         if (e != hipSuccess) return (int)e;
     }
@@ -654,6 +679,7 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     p.A = (const half_t*)A; p.B = (const half_t*)B; p.C = (half_t*)C; p.ws = (float*)ws;
     p.M = M; p.N = N; p.K = K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
     p.tiles_m = (M + BM - 1) / BM; p.tiles_n = (N + BN - 1) / BN;
+    p.splits = split_factor(M, N, K);
     return launch<0>(p, ws, ws_bytes, s);
 }
 
@@ -671,6 +697,7 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
     p.M = (int)M; p.N = OC; p.K = (int)K; p.lda = 0; p.ldb = (int)K; p.ldc = OC;
     p.tiles_m = (int)((M + BM - 1) / BM); p.tiles_n = (OC + BN - 1) / BN;
     p.a_bytes = (unsigned)xbytes;
+    p.splits = split_factor(M, OC, K);
     p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M};
     // a K tile inside one filter tap (and a tap mask that fits 32 bits) takes the scalar-tap gather
     if (IC % BK == 0 && kH * kW <= 32) return launch<2>(p, ws, ws_bytes, s);

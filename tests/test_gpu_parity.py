@@ -86,8 +86,11 @@ FP16_CONFIGS = [(2, 256, 256, 128, 128, 64), (2, 256, 256, 64, 128, 64), (2, 128
 @pytest.mark.parametrize("cfg", FP16_CONFIGS)
 @pytest.mark.parametrize("splitk", [0, 1])
 def test_gemm_f16_vs_oracle(cfg, splitk):
+    if splitk and cfg[0] not in b16.SPLITK_STAGES_LIST:
+        pytest.skip("split-K libraries are built for the two-stage ring only")
     lib = load(b16.kernel_library("gemm_splitK" if splitk else "gemm", *cfg))
-    for (M, N, K) in [(256, 256, 256), (300, 200, 136), (1, 7, 8), (513, 1025, 72), (1024, 1024, 1024)]:
+    for (M, N, K) in [(256, 256, 256), (300, 200, 136), (1, 7, 8), (513, 1025, 72), (1024, 1024, 1024), (130, 260, 4096),
+                      (77, 90, 520), (64, 66, 2048)]:
         A, B = seeded_inputs.gemm_operands(M, N, K, np.float16)
         got = run_gemm_f16(lib, A, B)
         want = O.hgemm_f32acc(A, B)
@@ -189,7 +192,8 @@ def test_gemm_f16_rejects_bad_arguments():
     with pytest.raises(HelixError):
         lib.gemm(p, p, C.data_ptr(), 64, 64, 60, 64, 64, 64)
     sk = load(b16.kernel_library("gemm_splitK", 2, 128, 128, 64, 64, 64))
-    assert sk.workspace_bytes(64, 64, 64) == 2 * 64 * 64 * 4
+    assert sk.workspace_bytes(64, 64, 64) == 2 * 64 * 64 * 4           # one K tile: the minimum 2-way split
+    assert sk.workspace_bytes(64, 64, 4096) == 8 * 64 * 64 * 4         # one output tile, long K: 8-way
     assert sk.gemm(p, p, C.data_ptr(), 64, 64, 64, 64, 64, 64, 0, 0, check=False) == HELIX_ERR_WORKSPACE
 
 

@@ -61,7 +61,7 @@ def test_fp16_library_names():
     assert b16.library_for_key((0, 16, 128, 0, 0, 1, 0)).endswith("build/bin_fp16/libgemv_splitK.so")
     src, out, defines = b16.compile_job("gemm_splitK", 2, 128, 64, 64, 32, 64)
     assert src.endswith("src_template/MI355X_FP16/gemm.hip")
-    assert defines == {"SPLIT_K": 2, "LDS_STAGES": 2, "BLOCK_ROWS": 128, "BLOCK_COLS": 64, "WAVE_ROWS": 64,
+    assert defines == {"SPLIT_K": 8, "LDS_STAGES": 2, "BLOCK_ROWS": 128, "BLOCK_COLS": 64, "WAVE_ROWS": 64,
                        "WAVE_COLS": 32, "BLOCK_K": 64}
     cmd = helix_runtime.compile_command(src, out, defines)
     assert "--offload-arch=gfx950" in cmd and "-DBLOCK_ROWS=128" in cmd and "-shared" in cmd
@@ -93,7 +93,13 @@ def test_fp16_cost_model_hand_cases():
     assert g16.cost_model(d, 300, 300, K) == (2, 128, 128, 64, 64, 0, 64)
     # round time scales with K
     assert g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 4096, 4096, K // 2) == pytest.approx(2.0)
-    # split-K doubles the blocks (reference: * (k[5] + 1)) and halves the K walk
+    # split-K multiplies the blocks (reference: * (k[5] + 1); here 2..8 ways, as many as fill 256 CUs) and
+    # divides the K walk
+    assert g16.split_factor((2, 128, 128, 64, 64, 1, 64), 128, 128, 8192) == 8
+    assert g16.split_factor((2, 128, 128, 64, 64, 1, 64), 1024, 1024, 8192) == 4
+    assert g16.split_factor((2, 128, 128, 64, 64, 1, 64), 8192, 8192, 8192) == 2
+    assert g16.split_factor((2, 128, 128, 64, 64, 1, 64), 128, 128, 192) == 2
+    assert g16.split_factor((2, 128, 128, 64, 64, 0, 64), 128, 128, 8192) == 1
     c0 = g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 128, 128, 8192)
     c1 = g16.config_cost((2, 128, 128, 64, 64, 1, 64), 1.0, 128, 128, 8192)
     assert c1 < c0
