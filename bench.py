@@ -20,6 +20,7 @@ sys.path.insert(0, os.path.join(ROOT, "helix_amd", "scripts"))
 os.chdir(ROOT)
 
 SIZE = 8192
+MEASURED_TRAFFIC_BYTES = 1.746e9   # 1.612e9 fetched + 1.342e8 written per 8192^3 launch (rocprofv3 --pmc)
 
 
 def autotune(prof_keys, M, N, K):
@@ -152,9 +153,14 @@ def main():
     kern_s = lib.gemm_timed(A.data_ptr(), Bt.data_ptr(), C.data_ptr(), M, N, K, K, K, N, ws.data_ptr(), wsb, stream,
                             warmup=2, iters=args.steps)
     achieved = flops / kern_s / 1e12
+    # HBM-side bytes per launch of the 256 x 256-tile kernels at this size, from the FETCH_SIZE / WRITE_SIZE
+    # counter runs scaled by a 1 GiB copy (profiles/gemm_f16_8192_pmc.md); not measurable from inside this run
+    traffic = MEASURED_TRAFFIC_BYTES if (best[1], best[2]) == (256, 256) else None
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": FP16_MFMA_FLOPS / 1e12, "unit": "TFLOP/s",
-                "frac": round(achieved * 1e12 / FP16_MFMA_FLOPS, 4), "traffic": None,
-                "kernel": "helix_gemm_f16_kernel<false>", "kernel_avg_us": round(kern_s * 1e6, 2)}
+                "frac": round(achieved * 1e12 / FP16_MFMA_FLOPS, 4), "traffic": traffic,
+                "kernel": "helix_gemm_f16_kernel<0, %d, %d, %d, %d, %d, %d, 1>" % (best[0], best[1], best[2], best[3],
+                                                                                  best[4], best[6]),
+                "kernel_avg_us": round(kern_s * 1e6, 2)}
 
     # ---- spot check of the timed result against torch's FP32 matmul on a slice ------------------------------
     ref = A[:256].float() @ Bt[:256].float().t()
