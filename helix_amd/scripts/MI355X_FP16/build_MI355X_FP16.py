@@ -7,8 +7,10 @@ names modulo the backend tag.  Differences that follow from the target:
   * output is build/bin_fp16/lib<kernel>_<params>.so exporting the C ABI of include/helix_abi.h instead of
     an executable; the convolution path lives in the same library as the GEMM of each configuration
     (implicit GEMM), so there is no im2col artifact;
-  * wave tiles are multiples of the 32x32 MFMA tile, K_STAGE becomes LDS_STAGES, and BLOCK_K is a
-    template parameter too (it is fixed to 32 in the reference, gemm.cu:77);
+  * wave tiles are multiples of 32x32 (2x2 of the 16x16x32 MFMA tile), K_STAGE becomes K_STAGES (the
+    pipeline holds the K tile being multiplied in LDS and one more on its way through registers: 2 is the
+    only depth the gfx950 template implements), and BLOCK_K is a template parameter too (it is fixed to 32
+    in the reference, gemm.cu:77);
   * compiles run in parallel worker threads instead of one os.system at a time.
 """
 import os
@@ -18,17 +20,30 @@ from utils.helix_runtime import SRC_ROOT, bin_dir, compile_many
 
 root_path = os.getcwd()
 
-LDS_STAGES_LIST = [2, 3, 4]
+K_STAGES_LIST = [2]
 SPLITK_MAX = 8              # a split-K library partitions K 2 .. 8 ways, chosen per problem
-SPLITK_STAGES_LIST = [2]    # split-K variants are built for the two-stage ring only (tiny M x N problems)
+SPLITK_STAGES_LIST = [2]    # pipeline depths a split-K variant is built for
 WAVE_TILE_LIST = [32, 64, 128]
 BLOCK_SCALE_LIST = [1, 2, 4]
-BLOCK_K_LIST = [32, 64]
+BLOCK_K_LIST = [64, 128]
 LDS_LIMIT = 160 * 1024
+VGPR_FILE = 512             # registers per lane of one SIMD (arch + accumulation), shared by its resident waves
+
+
+def vgpr_estimate(block_rows, block_cols, wave_rows, wave_cols, block_k):
+    """Registers per lane the kernel keeps live in its main loop: FP32 accumulators, the double-buffered
+    fragments of the operand with more 16-row fragments, the 4-deep window of the other one, the staging
+    registers of one K tile, and about 16 for addresses."""
+    threads = 64 * (block_rows // wave_rows) * (block_cols // wave_cols)
+    tm, tn = wave_rows // 16, wave_cols // 16
+    acc = wave_rows * wave_cols // 64
+    frags = 2 * max(tm, tn) * 4 + 4 * 4
+    staging = (block_rows + block_cols) * (block_k // 8) // threads * 4
+    return acc + frags + staging + 16
 
 
 def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, wave_rows, wave_cols,
-                    block_k=64, lds_stages=2):
+                    block_k=64, k_stages=2):
     # the reference's four rules (build_Ampere_FP16.py:30-39)
     if block_rows_scale == 4 and block_cols_scale == 4:
         return False
@@ -38,10 +53,10 @@ def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, 
         return False
     if block_cols == block_rows * 16 or block_rows == block_cols * 16:
         return False
-    # gfx950 resources: LDS ring, FP32 accumulators per lane, even split of the tile copy over threads
-    if lds_stages * (block_rows + block_cols) * block_k * 2 > LDS_LIMIT:
+    # gfx950 resources: two LDS stages, even split of the tile copy over threads, registers
+    if k_stages != 2:
         return False
-    if wave_rows * wave_cols // 64 > 256:
+    if 2 * (block_rows + block_cols) * block_k * 2 > LDS_LIMIT:
         return False
     threads = 64 * block_rows_scale * block_cols_scale
     chunks_per_row = block_k // 8
@@ -49,17 +64,15 @@ def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, 
         return False
     if threads % chunks_per_row:
         return False
-    # copy instructions of the later ring stages stay in flight while the wave waits for the next one:
-    # the hardware's outstanding-load counter holds 6 bits
-    copies_per_tile = (block_rows + block_cols) * chunks_per_row // threads
-    if (lds_stages - 1) * copies_per_tile > 63:
+    waves_per_simd = (threads // 64 + 3) // 4
+    if vgpr_estimate(block_rows, block_cols, wave_rows, wave_cols, block_k) > VGPR_FILE // waves_per_simd:
         return False
     return True
 
 
 def iter_configs():
-    """Yields (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in build order."""
-    for LDS_STAGES in LDS_STAGES_LIST:
+    """Yields (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in build order."""
+    for K_STAGES in K_STAGES_LIST:
         for WAVE_ROWS in WAVE_TILE_LIST:
             for WAVE_COLS in WAVE_TILE_LIST:
                 for BLOCK_ROWS_SCALE in BLOCK_SCALE_LIST:
@@ -68,24 +81,24 @@ def iter_configs():
                             BLOCK_ROWS = BLOCK_ROWS_SCALE * WAVE_ROWS
                             BLOCK_COLS = BLOCK_COLS_SCALE * WAVE_COLS
                             if not is_valid_config(BLOCK_ROWS_SCALE, BLOCK_COLS_SCALE, BLOCK_ROWS, BLOCK_COLS,
-                                                   WAVE_ROWS, WAVE_COLS, BLOCK_K, LDS_STAGES):
+                                                   WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES):
                                 continue
-                            yield (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K)
+                            yield (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K)
 
 
-def kernel_library(kernel_name, lds_stages=None, block_rows=None, block_cols=None, wave_rows=None, wave_cols=None,
+def kernel_library(kernel_name, k_stages=None, block_rows=None, block_cols=None, wave_rows=None, wave_cols=None,
                    block_k=None):
     """Path of the shared library of one configuration (same naming scheme as the reference's
     executables, build_Ampere_FP16.py:13-27, plus the BLOCK_K field)."""
     output_name = kernel_name
-    for v in (lds_stages, block_rows, block_cols, wave_rows, wave_cols, block_k):
+    for v in (k_stages, block_rows, block_cols, wave_rows, wave_cols, block_k):
         if v is not None:
             output_name += f"_{v}"
     return f"{bin_dir('fp16')}/lib{output_name}.so"
 
 
 def library_for_key(key):
-    """prof-dict key -> library path.  key = (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS,
+    """prof-dict key -> library path.  key = (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS,
     splitK flag, BLOCK_K); key[0] == 0 marks the GEMV kernels, as in the reference
     (scripts/Ampere_FP16/Ampere_FP16_gemm.py:435)."""
     if key[0] == 0:
@@ -93,7 +106,7 @@ def library_for_key(key):
     return kernel_library("gemm" if key[5] == 0 else "gemm_splitK", key[0], key[1], key[2], key[3], key[4], key[6])
 
 
-def compile_job(kernel_name, lds_stages=None, block_rows=None, block_cols=None, wave_rows=None, wave_cols=None,
+def compile_job(kernel_name, k_stages=None, block_rows=None, block_cols=None, wave_rows=None, wave_cols=None,
                 block_k=None):
     defines = {}
     src_name = kernel_name
@@ -103,8 +116,8 @@ def compile_job(kernel_name, lds_stages=None, block_rows=None, block_cols=None, 
     elif kernel_name == "gemv_splitK":
         src_name = "gemv"
         defines["SPLIT_K"] = 4
-    if lds_stages is not None:
-        defines["LDS_STAGES"] = lds_stages
+    if k_stages is not None:
+        defines["K_STAGES"] = k_stages
     if block_rows is not None:
         defines["BLOCK_ROWS"] = block_rows
     if block_cols is not None:
@@ -116,7 +129,7 @@ def compile_job(kernel_name, lds_stages=None, block_rows=None, block_cols=None, 
     if block_k is not None:
         defines["BLOCK_K"] = block_k
     src = f"{SRC_ROOT}/MI355X_FP16/{src_name}.hip"
-    out = kernel_library(kernel_name, lds_stages, block_rows, block_cols, wave_rows, wave_cols, block_k)
+    out = kernel_library(kernel_name, k_stages, block_rows, block_cols, wave_rows, wave_cols, block_k)
     return (src, out, defines)
 
 

@@ -8,7 +8,7 @@ import os
 from tqdm import tqdm
 
 from utils.helix_runtime import write_prof_dict
-from MI355X_FP16.build_MI355X_FP16 import (LDS_STAGES_LIST, WAVE_TILE_LIST, BLOCK_SCALE_LIST, BLOCK_K_LIST,
+from MI355X_FP16.build_MI355X_FP16 import (K_STAGES_LIST, WAVE_TILE_LIST, BLOCK_SCALE_LIST, BLOCK_K_LIST,
                                            is_valid_config, SPLITK_STAGES_LIST)
 from MI355X_FP16.profile_MI355X_FP16 import time_config, GEMV_KEYS, GEMV_SPLITK_KEYS
 
@@ -21,27 +21,27 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
 
     prof_dict = {}
     print("Start profiling MI355X FP16 GEMM kernel ...")
-    total = len(LDS_STAGES_LIST) * len(WAVE_TILE_LIST) ** 2 * len(BLOCK_K_LIST) * 2 + 2
+    total = len(K_STAGES_LIST) * len(WAVE_TILE_LIST) ** 2 * len(BLOCK_K_LIST) * 2 + 2
     with tqdm(total=total, desc="profiling") as pbar:
-        for LDS_STAGES in LDS_STAGES_LIST:
+        for K_STAGES in K_STAGES_LIST:
             for WAVE_ROWS in WAVE_TILE_LIST:
                 for WAVE_COLS in WAVE_TILE_LIST:
                     for BLOCK_K in BLOCK_K_LIST:
                         for splitK in (0, 1):
                             pbar.update(1)
-                            if splitK == 1 and LDS_STAGES not in SPLITK_STAGES_LIST:
+                            if splitK == 1 and K_STAGES not in SPLITK_STAGES_LIST:
                                 continue
-                            if not is_valid_config(1, 1, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K, LDS_STAGES):
+                            if not is_valid_config(1, 1, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES):
                                 continue
-                            cost = time_config((LDS_STAGES, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K))
+                            cost = time_config((K_STAGES, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K))
                             for BLOCK_ROWS_SCALE in BLOCK_SCALE_LIST:
                                 for BLOCK_COLS_SCALE in BLOCK_SCALE_LIST:
                                     BLOCK_ROWS = BLOCK_ROWS_SCALE * WAVE_ROWS
                                     BLOCK_COLS = BLOCK_COLS_SCALE * WAVE_COLS
                                     if not is_valid_config(BLOCK_ROWS_SCALE, BLOCK_COLS_SCALE, BLOCK_ROWS, BLOCK_COLS,
-                                                           WAVE_ROWS, WAVE_COLS, BLOCK_K, LDS_STAGES):
+                                                           WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES):
                                         continue
-                                    prof_dict[(LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, splitK,
+                                    prof_dict[(K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, splitK,
                                                BLOCK_K)] = float(cost) * BLOCK_ROWS_SCALE * BLOCK_COLS_SCALE
 
         for key in GEMV_KEYS + GEMV_SPLITK_KEYS:

@@ -53,10 +53,10 @@ def time_config(key, warmup=3, iters=10):
 
 def all_keys():
     keys = []
-    for (LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in iter_configs():
-        keys.append((LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 0, BLOCK_K))
-        if LDS_STAGES in SPLITK_STAGES_LIST:
-            keys.append((LDS_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 1, BLOCK_K))
+    for (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in iter_configs():
+        keys.append((K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 0, BLOCK_K))
+        if K_STAGES in SPLITK_STAGES_LIST:
+            keys.append((K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 1, BLOCK_K))
     keys.extend(GEMV_KEYS)
     keys.extend(GEMV_SPLITK_KEYS)
     return keys

@@ -12,20 +12,22 @@
 // Compile-time parameters (set with -D by the build script, one shared library per combination):
 //   BLOCK_ROWS x BLOCK_COLS   workgroup tile of C           (reference BLOCK_ROWS / BLOCK_COLS)
 //   WAVE_ROWS  x WAVE_COLS    tile of C owned by one wave64 (reference WARP_ROWS / WARP_COLS)
-//   BLOCK_K                   K extent of one LDS stage
-//   LDS_STAGES                LDS ring depth                (reference K_STAGE)
+//   BLOCK_K                   K extent of one LDS stage (64 or 128)
+//   K_STAGES                  K tiles in the pipeline: 2 = the tile being multiplied + one staged in
+//                             registers on its way to LDS, 3 = two staged      (reference K_STAGE)
 //   SPLIT_K                   1: each workgroup walks all of K.  > 1: K is partitioned over blockIdx.y into
 //                             2 .. SPLIT_K ranges, as many as it takes to give every compute unit a
 //                             workgroup (FP32 workspace + fixed-order reduction kernel)
 //
 // Kernel structure
-//   * one wave64 computes (WAVE_ROWS/32) x (WAVE_COLS/32) v_mfma_f32_32x32x16_f16 tiles; per 16-wide
-//     k step it reads one 16-byte fragment per 32 rows of A and of B from LDS (ds_read_b128).
-//   * global -> LDS uses gfx950's 128-bit direct-to-LDS buffer loads (DIRECT_TO_LDS=1, default): no
-//     staging registers, no ds_write; hardware bounds checking zero-fills rows beyond M / N and the K
-//     tail.  The copy of tile t+1 is issued after tile t's fragments are read and lands while tile t's
-//     MFMAs run; one wait + barrier per tile.  DIRECT_TO_LDS=0 keeps the register-staged variant
-//     (buffer_load -> VGPR -> ds_write_b128).
+//   * one wave64 computes (WAVE_ROWS/16) x (WAVE_COLS/16) v_mfma_f32_16x16x32_f16 tiles.  The 16x16x32
+//     shape does twice the K depth per accumulator access of the 32x32x16 one; on random data, where the
+//     chip runs against its power limit, MFMA-only loops measure 1.95 PFLOP/s with it against 1.69.
+//   * global -> registers (128-bit buffer loads; hardware bounds checking zero-fills rows beyond M / N and
+//     the K tail) -> LDS (ds_write_b128) -> fragments (ds_read_b128).  Two LDS stages; the loads of a tile
+//     are issued one or two tiles ahead and every memory instruction sits behind its own MFMA, evenly
+//     spread over the tile, so that the four waves of a workgroup never queue bursts on the CU's single
+//     address unit (a burst of 64 KiB behind a barrier costs more than the k-step it hides in).
 //   * LDS rows are BLOCK_K halves; 16-byte chunk c of row r is stored at chunk (c ^ key(r)), with
 //     key(r) = (r / rows_per_256B) mod chunks_per_row, so that 16 consecutive rows of one chunk column
 //     land in 16 different 16-byte bank groups (64 banks x 4 B): fragment reads and tile writes are
@@ -35,6 +37,8 @@
 //     GROUP_ROWS tile rows; each XCD's L2 then sees a compact patch of tiles sharing A and B panels.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "helix_abi.h"
 
@@ -53,8 +57,8 @@
 #ifndef BLOCK_K
 #define BLOCK_K 64
 #endif
-#ifndef LDS_STAGES
-#define LDS_STAGES 2
+#ifndef K_STAGES
+#define K_STAGES 2
 #endif
 #ifndef SPLIT_K
 #define SPLIT_K 1
@@ -62,24 +66,20 @@
 #ifndef GROUP_ROWS
 #define GROUP_ROWS 8
 #endif
-#ifndef DIRECT_TO_LDS
-#define DIRECT_TO_LDS 1
-#endif
 
 namespace {
 
 typedef _Float16 half_t;
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
 typedef int intx2 __attribute__((ext_vector_type(2)));
 
 constexpr int BM = BLOCK_ROWS, BN = BLOCK_COLS, WM = WAVE_ROWS, WN = WAVE_COLS, BK = BLOCK_K;
-constexpr int STAGES = LDS_STAGES, SPLITK = SPLIT_K;
+constexpr int STAGES = K_STAGES, SPLITK = SPLIT_K;
 constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN, NWAVES = WAVES_M * WAVES_N, NTHREADS = 64 * NWAVES;
-constexpr int TM = WM / 32, TN = WN / 32;      // MFMA tiles per wave
+constexpr int TM = WM / 16, TN = WN / 16;      // MFMA tiles per wave
 constexpr int KCH = BK / 8;                    // 16-byte chunks per LDS row
 constexpr int ROW_BYTES = BK * 2;
 constexpr int RP = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;  // rows per 256 bytes of LDS
@@ -87,24 +87,18 @@ constexpr int A_ITERS = BM * KCH / NTHREADS, B_ITERS = BN * KCH / NTHREADS;
 constexpr int ROWS_PER_ITER = NTHREADS / KCH;
 constexpr int A_STAGE_BYTES = BM * ROW_BYTES, B_STAGE_BYTES = BN * ROW_BYTES;
 constexpr int STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
-constexpr int RING_BYTES = STAGES * STAGE_BYTES;
+constexpr int RING_BYTES = 2 * STAGE_BYTES;
 // epilogue staging: one 32 x WAVE_COLS strip of halves per wave, rows padded by 16 bytes
 constexpr int STRIP_LD = WN * 2 + 16;
 constexpr int STRIP_BYTES = 32 * STRIP_LD;
 constexpr int LDS_BYTES = RING_BYTES > NWAVES * STRIP_BYTES ? RING_BYTES : NWAVES * STRIP_BYTES;
 
 static_assert(BM % WM == 0 && BN % WN == 0, "block tile must be a multiple of the wave tile");
-static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is built from 32x32 MFMA tiles");
-static_assert(BK % 16 == 0 && (KCH & (KCH - 1)) == 0 && KCH >= 2, "BLOCK_K must be 16 * 2^n");
+static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32 x 32");
+static_assert(BK == 64 || BK == 128, "BLOCK_K holds an even number of 32-wide MFMA k-steps: 64 or 128");
 static_assert(NTHREADS <= 1024 && NTHREADS % KCH == 0, "bad thread count");
 static_assert((BM * KCH) % NTHREADS == 0 && (BN * KCH) % NTHREADS == 0, "tile copy must divide evenly");
-#if DIRECT_TO_LDS
-static_assert(STAGES >= 2 && STAGES <= 4, "LDS ring depth must be 2..4");
-static_assert((BK / 16) % 2 == 0, "BLOCK_K must hold an even number of 16-wide MFMA k-steps");
-static_assert((STAGES - 1) * (A_ITERS + B_ITERS) <= 63, "too many copy instructions in flight for vmcnt");
-#else
-static_assert(STAGES == 2, "the register-staged variant implements the two-stage ring only");
-#endif
+static_assert(STAGES == 2, "K_STAGES: one K tile staged in registers behind the one in LDS");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
 static_assert(SPLITK >= 1 && SPLITK <= 8, "SPLIT_K out of range");
 
@@ -131,34 +125,79 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, un
 }
 
 constexpr int OOB_OFFSET = 0x7fffffff;  // byte offset beyond any buffer: the load returns zeros
-constexpr int KSTEPS = BK / 16;         // MFMA k-steps per K tile
-typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
-
-// s_waitcnt vmcnt(N): at most N buffer loads of this wave (also the direct-to-LDS ones) are still in flight
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
-    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
-}
-
-// 128-bit buffer descriptor as four dwords: base address (48 bits), stride 0, byte count, raw-buffer flags
-__device__ __forceinline__ intx4 raw_rsrc(const void* base, unsigned bytes) {
-    const unsigned long long a = (unsigned long long)base;
-    intx4 r = {(int)(unsigned)a, (int)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
-    return r;
-}
-
-// One 16-byte-per-lane direct-to-LDS buffer load: lane l's data lands at LDS byte (lds_addr + 16*l).
-// lds_addr must be wave-uniform (it is moved into M0); voff is the per-lane byte offset into the buffer.
-__device__ __forceinline__ void dma16(intx4 rsrc, unsigned lds_addr, int voff) {
-    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :
-                 : "s"(lds_addr), "v"(voff), "s"(rsrc)
-                 : "memory", "m0");
-}
+constexpr int KSTEPS = BK / 32;         // MFMA k-steps per K tile (2 or 4)
 
 __device__ __forceinline__ intx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) {
     return __builtin_bit_cast(intx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+}
+
+// ---- static instruction schedule of one K tile ---------------------------------------------------------
+// A K tile is G = KSTEPS * TM * TN MFMAs ("slots"), and every memory instruction of the tile is issued behind
+// one of them.  A 16x16x32 MFMA keeps the matrix pipe busy for 16 cycles, which leaves the wave room for
+// about two other instructions per slot before the pipe runs dry, so the instructions are dealt out as
+// evenly as the data dependences allow.  The operand with more fragments per k-step is "resident" (double
+// buffered by k-step), the other one is "streamed" (PD fragments ahead through 2*PD registers):
+//   * streamed fragment n+PD is read behind the first MFMA that uses fragment n           (slot n * T_RES);
+//   * resident fragment v of the next k-step is read half way between two of those  (slot s*NM + v*T_STR +
+//     T_STR/2); the next tile's first k-step is read in the PD * T_RES slots past the barrier;
+//   * the LDS write of copy slot idx goes to the least loaded slot of its share of the first WSLOTS slots,
+//     the global load that refills the same register to the least loaded later slot of its share of all G.
+constexpr bool RES_A = (TM > TN);              // resident operand: A if it has more fragments, else B
+constexpr int T_RES = RES_A ? TM : TN, T_STR = RES_A ? TN : TM;
+constexpr int NM = TM * TN;                    // MFMAs per k-step
+constexpr int G = KSTEPS * NM;                 // MFMAs per K tile
+constexpr int PD = T_STR < 2 ? T_STR : 2;      // read-ahead distance of the streamed operand, in fragments
+constexpr int AW = 2 * PD;                     // its register window
+constexpr int NSTR = KSTEPS * T_STR;           // streamed fragments per K tile
+constexpr int G_BAR = (NSTR - PD) * T_RES;     // slot in front of which the workgroup barrier sits
+constexpr int NV = A_ITERS + B_ITERS;          // copy slots (16 bytes per thread each) per K tile
+#ifdef WRITE_SLOTS
+constexpr int WSLOTS = WRITE_SLOTS;
+#else
+// LDS writes are kept to the first two thirds of the slots in front of the barrier, so that they have drained
+// when the barrier is reached
+constexpr int WSLOTS = (2 * G_BAR / 3) > 0 ? (2 * G_BAR / 3) : 1;
+#endif
+static_assert(NSTR % AW == 0, "streamed fragment window must divide the fragments of a tile");
+static_assert(WSLOTS >= 1 && WSLOTS <= G_BAR, "LDS writes must be issued in front of the barrier");
+
+struct Schedule {
+    int wslot[NV];   // slot of the LDS write of copy slot idx
+    int lslot[NV];   // slot of the global load that refills its register (>= wslot)
+};
+
+constexpr int res_read_slot(int s, int v) { return s * NM + v * T_STR + T_STR / 2; }      // k-step s+1, in tile
+constexpr int res_next_slot(int v) { return G_BAR + v * PD + (PD - 1); }                  // next tile, k-step 0
+
+constexpr Schedule make_schedule() {
+    Schedule sc{};
+    int cnt[G] = {};
+    for (int n = 0; n < NSTR; n++) cnt[n * T_RES]++;
+    for (int s = 0; s + 1 < KSTEPS; s++)
+        for (int v = 0; v < T_RES; v++) cnt[res_read_slot(s, v)]++;
+    for (int v = 0; v < T_RES; v++) cnt[res_next_slot(v)]++;
+    for (int idx = 0; idx < NV; idx++) {
+        const int lo = idx * WSLOTS / NV;
+        int hi = (idx + 1) * WSLOTS / NV;
+        if (hi <= lo) hi = lo + 1;
+        int best = lo;
+        for (int g = lo; g < hi; g++)
+            if (cnt[g] < cnt[best]) best = g;
+        sc.wslot[idx] = best;
+        cnt[best]++;
+    }
+    for (int idx = 0; idx < NV; idx++) {
+        int lo = idx * G / NV;
+        if (lo < sc.wslot[idx]) lo = sc.wslot[idx];
+        int hi = (idx + 1) * G / NV;
+        if (hi <= lo) hi = lo + 1;
+        int best = lo;
+        for (int g = lo; g < hi; g++)
+            if (cnt[g] <= cnt[best]) best = g;      // ties: the latest slot
+        sc.lslot[idx] = best;
+        cnt[best]++;
+    }
+    return sc;
 }
 
 // The tile parameters appear as (otherwise unused) template arguments so that every configuration's
@@ -277,10 +316,11 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     };
 
     // Byte offset (relative to the operand's buffer descriptor) of copy slot i for the K tile at k0, or
-    // OOB_OFFSET when the slot must read zeros (beyond K, conv padding, rows beyond M).
-    auto a_offset = [&](int i, int k0, bool tail, ConvTile ct) -> int {
+    // OOB_OFFSET when the slot must read zeros (conv padding, rows beyond M, and -- only for the first tile
+    // of the K range, which is the one that may be narrower than BLOCK_K -- columns beyond its width).
+    auto a_offset = [&](int i, int k0, bool narrow, int width, ConvTile ct) -> int {
         if (!CONV) {
-            return (tail && k0 + gch_a[i] * 8 >= p.K) ? OOB_OFFSET : voff_a[i];
+            return (narrow && gch_a[i] * 8 >= width) ? OOB_OFFSET : voff_a[i];
         } else if (MODE == 2) {
             return (cv_taps[i] & ct.tapbit) ? cv_base[i] + ct.soff : OOB_OFFSET;
         } else {
@@ -290,227 +330,195 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             const int kw = t % p.g.kW;
             const int kh = t / p.g.kW;
             const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
-            const bool ok = k < p.K && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W;
+            const bool ok = !(narrow && gch_a[i] * 8 >= width) && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 &&
+                            iw < p.g.W;
             return ok ? ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 2 : OOB_OFFSET;
         }
     };
-    auto b_offset = [&](int i, int k0, bool tail) -> int {
-        return (tail && k0 + gch_b[i] * 8 >= p.K) ? OOB_OFFSET : voff_b[i];
+    auto b_offset = [&](int i, bool narrow, int width) -> int {
+        return (narrow && gch_b[i] * 8 >= width) ? OOB_OFFSET : voff_b[i];
     };
 
-#if DIRECT_TO_LDS
-    // global -> LDS without passing through registers: each wave-wide load deposits 64 x 16 bytes at a
-    // wave-uniform LDS address (M0) in lane order.  The loads are issued from inline assembly so that
-    // the compiler does not serialise later LDS reads behind them; completion is tracked by hand with
-    // s_waitcnt vmcnt(n) before the workgroup barrier that publishes a stage.
-    const unsigned lds_base = (unsigned)(uintptr_t)(lds_ptr_t)smem;
-    const unsigned lds_wave = lds_base + (unsigned)wave * 1024u;
-    // copy slot `idx` (A slots first, then B slots) of the K tile at k0 into LDS stage `stage`
-    auto copy_slot = [&](int idx, int stage, int k0, bool tail, intx4 ra, intx4 rb, ConvTile ct) {
-        if (idx < A_ITERS) {
-            const int off = a_offset(idx, k0, tail, ct);
-            dma16(ra, lds_wave + (unsigned)(stage * STAGE_BYTES + idx * NTHREADS * 16), off);
-        } else {
-            const int i = idx - A_ITERS;
-            const int off = b_offset(i, k0, tail);
-            dma16(rb, lds_wave + (unsigned)(stage * STAGE_BYTES + A_STAGE_BYTES + i * NTHREADS * 16), off);
-        }
+    // global -> registers -> LDS.  Copy slot idx (A slots first, then B slots) of a K tile is one 16-byte
+    // buffer load per lane; hardware bounds checking zero-fills rows beyond M / N.
+    auto load_slot = [&](int idx, int k0, bool narrow, int width, __amdgpu_buffer_rsrc_t ra,
+                         __amdgpu_buffer_rsrc_t rb, ConvTile ct) -> intx4 {
+        if (idx < A_ITERS) return buf_load16(ra, a_offset(idx, k0, narrow, width, ct));
+        return buf_load16(rb, b_offset(idx - A_ITERS, narrow, width));
     };
-    auto rsrc_a = [&](int k0) -> intx4 {
-        return CONV ? raw_rsrc(baseA, bytesA) : raw_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
+    auto store_slot = [&](int idx, int stage, intx4 v) {
+        const int off = idx < A_ITERS ? idx * NTHREADS * 16 : A_STAGE_BYTES + (idx - A_ITERS) * NTHREADS * 16;
+        *(intx4*)(smem + stage * STAGE_BYTES + off + tid * 16) = v;
     };
-    auto rsrc_b = [&](int k0) -> intx4 { return raw_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u); };
-#else
-    intx4 stage_a[A_ITERS], stage_b[B_ITERS];
-    auto load_global = [&](int k0) {
-        const bool tail = (k0 + BK > p.K);
-        __amdgpu_buffer_rsrc_t rb = make_rsrc(baseB + k0, bytesB - (unsigned)k0 * 2u);
-        __amdgpu_buffer_rsrc_t ra = CONV ? make_rsrc(baseA, bytesA) : make_rsrc(baseA + k0, bytesA - (unsigned)k0 * 2u);
-#pragma unroll
-        for (int i = 0; i < B_ITERS; i++) stage_b[i] = buf_load16(rb, b_offset(i, k0, tail));
-        const ConvTile ct = conv_tile(k0);
-#pragma unroll
-        for (int i = 0; i < A_ITERS; i++) stage_a[i] = buf_load16(ra, a_offset(i, k0, tail, ct));
+    // descriptors of the K tile at k0; `live` false gives empty ones (every load returns zeros)
+    auto rsrc_a = [&](int k0, bool live) -> __amdgpu_buffer_rsrc_t {
+        const unsigned n = !live ? 0u : CONV ? bytesA : bytesA - (unsigned)k0 * 2u;
+        return make_rsrc(CONV ? baseA : baseA + k0, n);
     };
-    auto store_lds = [&](int stage) {
-        unsigned char* base = smem + stage * STAGE_BYTES + tid * 16;
-#pragma unroll
-        for (int i = 0; i < A_ITERS; i++) *(intx4*)(base + i * NTHREADS * 16) = stage_a[i];
-#pragma unroll
-        for (int i = 0; i < B_ITERS; i++) *(intx4*)(base + A_STAGE_BYTES + i * NTHREADS * 16) = stage_b[i];
+    auto rsrc_b = [&](int k0, bool live) -> __amdgpu_buffer_rsrc_t {
+        return make_rsrc(baseB + k0, live ? bytesB - (unsigned)k0 * 2u : 0u);
     };
-#endif
 
     // ---- fragment read geometry -----------------------------------------------------------------
-    // MFMA 32x32x16: lane l supplies row (l % 32), k = 8*(l/32) .. +7 of both operands.
-    const int frow = lane & 31, fhalf = lane >> 5;
+    // MFMA 16x16x32: lane l supplies row (l % 16), k = 8*(l/16) .. +7 of both operands, i.e. 16-byte chunk
+    // (4*s + l/16) of its row for k-step s.
+    const int frow = lane & 15, fq = lane >> 4;
     const int a_row = wave_m * WM + frow;
     const int b_row = wave_n * WN + frow;
     const int a_rd = a_row * ROW_BYTES, b_rd = A_STAGE_BYTES + b_row * ROW_BYTES;
     auto read_a = [&](const unsigned char* sb, int s, int i) -> half8 {
-        return *(const half8*)(sb + a_rd + i * 32 * ROW_BYTES + (((s * 2 + fhalf) ^ swz_key(a_row + i * 32)) << 4));
+        return *(const half8*)(sb + a_rd + i * 16 * ROW_BYTES + (((s * 4 + fq) ^ swz_key(a_row + i * 16)) << 4));
     };
     auto read_b = [&](const unsigned char* sb, int s, int j) -> half8 {
-        return *(const half8*)(sb + b_rd + j * 32 * ROW_BYTES + (((s * 2 + fhalf) ^ swz_key(b_row + j * 32)) << 4));
+        return *(const half8*)(sb + b_rd + j * 16 * ROW_BYTES + (((s * 4 + fq) ^ swz_key(b_row + j * 16)) << 4));
     };
 
-    floatx16 acc[TM][TN];
+    floatx4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-#pragma unroll
-            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+        for (int j = 0; j < TN; j++) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
 
-#if DIRECT_TO_LDS
-    // Software pipeline over K tiles with an LDS ring of STAGES stages (tile t lives in stage t % STAGES):
-    //   * during the MFMAs of k-step s the fragments of k-step s+1 are read from LDS (two register sets);
-    //   * before the last k-step of tile t the wave waits for its own copies of tile t+1 and the workgroup
-    //     barrier publishes that stage; at that point tile t's stage has been read completely (its last
-    //     fragments sit in registers), so the copy of tile t+STAGES is issued into it during the last
-    //     k-step, next to the reads of tile t+1's first fragments.  A copy therefore has a whole K tile
-    //     (STAGES-1 of them for deeper rings) to land before anyone waits for it.
-    // Every MFMA is followed by its share of the LDS reads / copy instructions and a scheduling fence, so
-    // the matrix pipe always has the next MFMA queued while the memory instructions issue in its shadow.
-    constexpr int NM = TM * TN;                    // MFMAs per k-step
-    constexpr int NR = TM + TN;                    // fragment reads per k-step
-    constexpr int NV = A_ITERS + B_ITERS;          // copy instructions per K tile
-    constexpr int RPM = (NR + NM - 1) / NM;        // reads issued behind each MFMA
-    constexpr int VPM = (NV + NM - 1) / NM;        // copies issued behind each MFMA (last k-step only)
-    half8 fa[2][TM], fb[2][TN];
+    // Software pipeline over K tiles.  Tile t is multiplied from LDS stage t % 2 while
+    //   * the staging registers that hold tile t+1 (loaded R tiles ago) are written to the other stage with
+    //     ds_write_b128 and each register is refilled with the same slot of tile t+1+R, so a global load has
+    //     R whole K tiles to land;
+    //   * fragments are read ahead of the MFMAs that use them: the operand with more fragments per k-step
+    //     (the "resident" one) is double-buffered by k-step and read one k-step ahead, the other one is
+    //     streamed through a small rotating set of registers, PD fragments ahead;
+    //   * one workgroup barrier per tile, placed between the last fragment read of tile t and the first one
+    //     of tile t+1 (PD streamed fragments before the end of the tile).  It publishes tile t+1, whose LDS
+    //     writes were all issued -- and had time to drain -- earlier in the tile, and it frees stage t % 2.
+    // Every MFMA is followed by its share of the memory instructions and a scheduling fence: the matrix pipe
+    // always has the next MFMA queued while the memory instructions issue in its shadow.
+    constexpr Schedule sched = make_schedule();
+    half8 fr[2][T_RES], fs[AW];
+    intx4 st[NV];
 
-    // fragment read order: a[0], b[0..TN-1], a[1..TM-1] -- the order the MFMAs below first need them
-    auto read_frag = [&](int idx, int set, const unsigned char* sb, int step) {
-        if (idx == 0) fa[set][0] = read_a(sb, step, 0);
-        else if (idx <= TN) fb[set][idx - 1] = read_b(sb, step, idx - 1);
-        else fa[set][idx - TN] = read_a(sb, step, idx - TN);
+    auto read_res = [&](const unsigned char* sb, int s, int v) -> half8 {
+        return RES_A ? read_a(sb, s, v) : read_b(sb, s, v);
+    };
+    auto read_str = [&](const unsigned char* sb, int s, int u) -> half8 {
+        return RES_A ? read_b(sb, s, u) : read_a(sb, s, u);
     };
 
+    // K tiles: when the K range is not a multiple of BLOCK_K the narrow tile comes first (tile 0 covers
+    // `first_w` columns, every later tile BLOCK_K), so that only the prologue's loads need a column mask
+    const int first_w = ((k_end - k_begin) % BK) ? ((k_end - k_begin) % BK) : BK;
+    auto tile_k0 = [&](int t) -> int { return t == 0 ? k_begin : k_begin + first_w + (t - 1) * BK; };
+
     if (ktiles > 0) {
-        // prologue: tiles 0 .. STAGES-1 in flight, tile 0 complete and published
+        // prologue: tile 0 into the staging registers and on to LDS, the registers refilled with tile 1
+        {
+            const __amdgpu_buffer_rsrc_t ra = rsrc_a(k_begin, true), rb = rsrc_b(k_begin, true);
+            const ConvTile ct = conv_tile(k_begin);
 #pragma unroll
-        for (int t = 0; t < STAGES; t++) {
-            if (t < ktiles) {
-                const int k0 = k_begin + t * BK;
-                const bool tail = (k0 + BK > p.K);
-                const intx4 ra = rsrc_a(k0), rb = rsrc_b(k0);
-                const ConvTile ct = conv_tile(k0);
+            for (int idx = 0; idx < NV; idx++) st[idx] = load_slot(idx, k_begin, true, first_w, ra, rb, ct);
+        }
+        {
+            const int k0 = tile_k0(1);
+            const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0, 1 < ktiles), rb = rsrc_b(k0, 1 < ktiles);
+            const ConvTile ct = conv_tile(k0);
 #pragma unroll
-                for (int idx = 0; idx < NV; idx++) copy_slot(idx, t, k0, tail, ra, rb, ct);
+            for (int idx = 0; idx < NV; idx++) {
+                store_slot(idx, 0, st[idx]);
+                st[idx] = load_slot(idx, k0, false, BK, ra, rb, ct);
             }
         }
-        // the copies complete in issue order: allow the later tiles' copies to stay in flight
-        if (ktiles >= STAGES) wait_vmcnt<(STAGES - 1) * NV>(); else wait_vmcnt<0>();
         __syncthreads();
+        // first fragments of tile 0, in the order in which the loop reads those of the next tile past its
+        // barrier: the compiler's wait counts at the loop head are the merge of both paths
 #pragma unroll
-        for (int idx = 0; idx < NR; idx++) read_frag(idx, 0, smem, 0);
+        for (int g = G_BAR; g < G; g++) {
+            if (g % T_RES == 0) {
+                const int n = g / T_RES + PD - NSTR;
+                fs[n % AW] = read_str(smem, n / T_STR, n % T_STR);
+            }
+#pragma unroll
+            for (int r = 0; r < T_RES; r++)
+                if (res_next_slot(r) == g) fr[0][r] = read_res(smem, 0, r);
+        }
     }
 
-    int stage_cur = 0;
-    for (int kt = 0; kt < ktiles; kt++) {
-        const unsigned char* sb = smem + stage_cur * STAGE_BYTES;
-        const int stage_nxt = (stage_cur + 1 == STAGES) ? 0 : stage_cur + 1;
-        const int kt_cpy = kt + STAGES;            // tile copied into stage_cur once tile kt has been read
-        const int k0c = k_begin + kt_cpy * BK;
-        const bool tailc = (k0c + BK > p.K);
-        // past the last tile the copy still issues, with empty descriptors: it writes zeros into a stage
-        // nobody reads again, which keeps the loop body free of branches
-        intx4 ra = rsrc_a(k0c), rb = rsrc_b(k0c);
-        if (kt_cpy >= ktiles) { ra[2] = 0; rb[2] = 0; }
+    // Slots [LO, HI) of K tile kt, multiplied from LDS stage `stage`.
+    auto tile_part = [&](auto lo_c, auto hi_c, int kt, int stage) {
+        constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
+        const unsigned char* sb = smem + stage * STAGE_BYTES;
+        const unsigned char* sb_nxt = smem + (stage ^ 1) * STAGE_BYTES;
+        const int kt_ld = kt + 2;                  // tile loaded into the staging registers once they are written
+        const int k0c = tile_k0(kt_ld);
+        // past the last tile the loads still issue, with empty descriptors, which keeps the body branch-free
+        const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0c, kt_ld < ktiles), rb = rsrc_b(k0c, kt_ld < ktiles);
         const ConvTile ctc = conv_tile(k0c);
-
 #pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            const int cur = s & 1, nxt = cur ^ 1;
-            const bool last = (s == KSTEPS - 1);
-            if (last) {
-                // tile kt+1 must be complete in LDS before its first fragments are read; the copies of
-                // tiles kt+2 .. kt+STAGES-1 (issued later) may stay in flight
-                __builtin_amdgcn_sched_barrier(0);
-                if (STAGES > 2 && kt + STAGES - 1 < ktiles) wait_vmcnt<(STAGES - 2) * NV>(); else wait_vmcnt<0>();
-                __syncthreads();
-                __builtin_amdgcn_sched_barrier(0);
+        for (int n = LO / T_RES; n < (HI + T_RES - 1) / T_RES; n++) {   // streamed fragment n: k-step s, index u
+#pragma unroll
+          for (int v = 0; v < T_RES; v++) {                             // resident fragment v
+            const int g = n * T_RES + v;                                // slot
+            if (g < LO || g >= HI) continue;
+            const int s = n / T_STR, u = n % T_STR;
+            if (RES_A) acc[v][u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fs[n % AW], fr[s & 1][v], acc[v][u], 0, 0, 0);
+            else acc[u][v] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fr[s & 1][v], fs[n % AW], acc[u][v], 0, 0, 0);
+            // streamed fragment n+PD, behind the first MFMA of fragment n (past the barrier: the next tile's)
+            if (v == 0) {
+                const int n2 = n + PD;
+                if (n2 < NSTR) fs[n2 % AW] = read_str(sb, n2 / T_STR, n2 % T_STR);
+                else fs[n2 % AW] = read_str(sb_nxt, (n2 - NSTR) / T_STR, (n2 - NSTR) % T_STR);
             }
-            const unsigned char* rd_base = last ? smem + stage_nxt * STAGE_BYTES : sb;
-            const int rd_step = last ? 0 : s + 1;
+            // resident fragments of the next k-step, or of the next tile's first k-step past the barrier
+            // (after the last tile these reads fetch an unused stage; their values are never consumed)
 #pragma unroll
-            for (int m = 0; m < NM; m++) {
-                const int i = m / TN, j = m % TN;
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
-                // (after the last tile these reads fetch an unused stage; their values are never consumed)
-#pragma unroll
-                for (int r = 0; r < RPM; r++)
-                    if (m * RPM + r < NR) read_frag(m * RPM + r, nxt, rd_base, rd_step);
-                if (last) {
-#pragma unroll
-                    for (int v = 0; v < VPM; v++)
-                        if (m * VPM + v < NV) copy_slot(m * VPM + v, stage_cur, k0c, tailc, ra, rb, ctc);
-                }
-                __builtin_amdgcn_sched_barrier(0);
+            for (int r = 0; r < T_RES; r++) {
+                if (s + 1 < KSTEPS && res_read_slot(s, r) == g) fr[(s + 1) & 1][r] = read_res(sb, s + 1, r);
+                if (res_next_slot(r) == g) fr[0][r] = read_res(sb_nxt, 0, r);
             }
+            // LDS writes of the staged tile and the refills of their registers
+#pragma unroll
+            for (int idx = 0; idx < NV; idx++) {
+                if (sched.wslot[idx] == g) store_slot(idx, stage ^ 1, st[idx]);
+                if (sched.lslot[idx] == g) st[idx] = load_slot(idx, k0c, false, BK, ra, rb, ctc);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
-        stage_cur = stage_nxt;
-    }
-#else
-    if (ktiles > 0) {
-        load_global(k_begin);
-        store_lds(0);
-    }
-    __syncthreads();
-
+    };
+    constexpr std::integral_constant<int, 0> c_0{};
+    constexpr std::integral_constant<int, G_BAR> c_bar{};
+    constexpr std::integral_constant<int, G> c_end{};
+    int stage = 0;
     for (int kt = 0; kt < ktiles; kt++) {
-        const int cur = kt & 1;
-        const bool more = (kt + 1 < ktiles);
-        if (more) load_global(k_begin + (kt + 1) * BK);
-
-        const unsigned char* sb = smem + cur * STAGE_BYTES;
-#pragma unroll
-        for (int s = 0; s < KSTEPS; s++) {
-            half8 af[TM], bf[TN];
-#pragma unroll
-            for (int i = 0; i < TM; i++) af[i] = read_a(sb, s, i);
-#pragma unroll
-            for (int j = 0; j < TN; j++) bf[j] = read_b(sb, s, j);
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bf[j], af[i], acc[i][j], 0, 0, 0);
-        }
-
-        if (more) store_lds(cur ^ 1);
+        tile_part(c_0, c_bar, kt, stage);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        tile_part(c_bar, c_end, kt, stage);
+        stage ^= 1;
     }
-#endif
 
     // ---- epilogue ---------------------------------------------------------------------------------
     // The MFMAs were issued with the B fragment as the first operand, so accumulator tile (i, j) holds the
-    // transposed 32x32 block: lane l owns tile row m = l % 32 and, in registers 4g..4g+3, the four
-    // consecutive tile columns n = 8g + 4*(l/32) + {0,1,2,3}.
-    const int m_l = lane & 31, n_l = (lane >> 5) * 4;
+    // transposed 16x16 block: lane l owns tile row m = l % 16 and the four consecutive tile columns
+    // n = 4*(l/16) + {0,1,2,3}.
+    const int m_l = lane & 15, n_l = (lane >> 4) * 4;
     if (SPLITK > 1) {
         // FP32 partial sums: four consecutive columns per lane, one 16-byte store where that is aligned
         const bool vec_ok = (p.N % 4 == 0);
 #pragma unroll
         for (int i = 0; i < TM; i++) {
-            const int row = m0 + wave_m * WM + i * 32 + m_l;
+            const int row = m0 + wave_m * WM + i * 16 + m_l;
 #pragma unroll
             for (int j = 0; j < TN; j++) {
+                const int col = n0 + wave_n * WN + j * 16 + n_l;
+                if (row < p.M) {
+                    float* dst = p.ws + ((size_t)blockIdx.y * p.M + row) * p.N + col;
+                    if (vec_ok && col + 4 <= p.N) {
+                        *(floatx4*)dst = acc[i][j];
+                    } else {
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const int col = n0 + wave_n * WN + j * 32 + g * 8 + n_l;
-                    if (row < p.M) {
-                        float* dst = p.ws + ((size_t)blockIdx.y * p.M + row) * p.N + col;
-                        if (vec_ok && col + 4 <= p.N) {
-                            floatx4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                            *(floatx4*)dst = v;
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; e++)
-                                if (col + e < p.N) dst[e] = acc[i][j][4 * g + e];
-                        }
+                        for (int e = 0; e < 4; e++)
+                            if (col + e < p.N) dst[e] = acc[i][j][e];
                     }
                 }
             }
@@ -519,9 +527,6 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         // FP16 result through LDS: each wave rounds a 32 x WAVE_COLS strip into its private LDS region
         // (8-byte writes), reads it back row-contiguous and stores 16 bytes per lane, so a store
         // instruction covers whole 2*WAVE_COLS-byte row segments.
-#if DIRECT_TO_LDS
-        wait_vmcnt<0>();   // the (empty) copies issued behind the last tiles still write zeros into the ring
-#endif
         __syncthreads();   // every wave is done reading the ring; the strips reuse its memory
         unsigned char* strip = smem + wave * STRIP_BYTES;
         // widest store the row stride and base address allow: 8, 4, 2 or 1 halves at a time
@@ -529,14 +534,14 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         const int vec = (valign == 0) ? 8 : (valign & 3) == 0 ? 4 : (valign & 1) == 0 ? 2 : 1;
         constexpr int CPR = WN / 8;                    // 16-byte chunks per strip row
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
+        for (int ii = 0; ii < TM / 2; ii++) {
 #pragma unroll
-            for (int j = 0; j < TN; j++) {
+            for (int hh = 0; hh < 2; hh++) {
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    half4 h = {(half_t)acc[i][j][4 * g], (half_t)acc[i][j][4 * g + 1], (half_t)acc[i][j][4 * g + 2],
-                               (half_t)acc[i][j][4 * g + 3]};
-                    *(half4*)(strip + m_l * STRIP_LD + (j * 32 + g * 8 + n_l) * 2) = h;
+                for (int j = 0; j < TN; j++) {
+                    const floatx4 a = acc[ii * 2 + hh][j];
+                    half4 h = {(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3]};
+                    *(half4*)(strip + (hh * 16 + m_l) * STRIP_LD + (j * 16 + n_l) * 2) = h;
                 }
             }
             __builtin_amdgcn_wave_barrier();   // same-wave LDS traffic stays in program order
@@ -545,7 +550,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
                 const int idx = t * 64 + lane;
                 const int r = idx / CPR, ch = idx % CPR;
                 const intx4 v = *(const intx4*)(strip + r * STRIP_LD + ch * 16);
-                const int row = m0 + wave_m * WM + i * 32 + r;
+                const int row = m0 + wave_m * WM + ii * 32 + r;
                 const int col = n0 + wave_n * WN + ch * 8;
                 if (row < p.M && col < p.N) {
                     half_t* dst = p.C + (size_t)row * p.ldc + col;
@@ -599,8 +604,8 @@ inline const char* info_json() {
     static bool done = false;
     if (!done) {
         snprintf(buf, sizeof(buf),
-                 "{\"family\": \"gemm_f16\", \"arch\": \"gfx950\", \"mfma\": \"v_mfma_f32_32x32x16_f16\", "
-                 "\"lds_stages\": %d, \"block_rows\": %d, \"block_cols\": %d, \"wave_rows\": %d, \"wave_cols\": %d, "
+                 "{\"family\": \"gemm_f16\", \"arch\": \"gfx950\", \"mfma\": \"v_mfma_f32_16x16x32_f16\", "
+                 "\"k_stages\": %d, \"block_rows\": %d, \"block_cols\": %d, \"wave_rows\": %d, \"wave_cols\": %d, "
                  "\"block_k\": %d, \"split_k\": %d, \"threads\": %d, \"lds_bytes\": %d, "
                  "\"layout_a\": \"M x K row-major f16\", \"layout_b\": \"N x K row-major f16\", "
                  "\"layout_c\": \"M x N row-major f16\", \"accumulate\": \"f32\", "

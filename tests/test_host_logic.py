@@ -22,8 +22,8 @@ from MI355X_FP32 import profile_MI355X_FP32 as p32
 from MI355X_FP32 import MI355X_FP32_gemm as g32
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-N_FP16_CONFIGS = 316   # 112 two-stage + 108 three-stage + 96 four-stage points of the FP16 template space
-N_FP16_SPLITK = 112    # split-K variants exist for the two-stage ring only
+N_FP16_CONFIGS = 106   # points of the FP16 template space (tile x wave tile x BLOCK_K) that fit LDS and registers
+N_FP16_SPLITK = 106    # every point also has a split-K variant
 
 
 # ---- enumeration ----------------------------------------------------------------------------------
@@ -35,7 +35,11 @@ def test_fp16_reference_validity_rules():
     assert not b16.is_valid_config(1, 4, 16, 256, 16, 64)             # block aspect 16x
     assert b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 2)
     # gfx950 resource rules
-    assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 128, 3)  # 3 x 512 x 128 x 2 B > 160 KiB of LDS
+    assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 128, 2)  # 2 x 512 x 128 x 2 B > 160 KiB of LDS
+    assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 3)   # only the two-tile pipeline exists
+    assert b16.is_valid_config(2, 4, 256, 256, 128, 64, 64, 2)        # 8 waves x 256 registers
+    assert b16.vgpr_estimate(256, 256, 128, 128, 64) == 256 + 80 + 64 + 16
+    assert b16.vgpr_estimate(256, 256, 128, 64, 64) == 128 + 80 + 32 + 16      # exactly the 256 of two waves per SIMD
 
 
 def test_fp16_template_space():
@@ -43,10 +47,10 @@ def test_fp16_template_space():
     assert len(cfgs) == N_FP16_CONFIGS and len(set(cfgs)) == N_FP16_CONFIGS
     for (st, br, bc, wr, wc, bk) in cfgs:
         assert br % wr == 0 and bc % wc == 0 and br <= 256 and bc <= 256
-        assert st * (br + bc) * bk * 2 <= 160 * 1024
+        assert st == 2 and bk in (64, 128) and 2 * (br + bc) * bk * 2 <= 160 * 1024
         threads = 64 * (br // wr) * (bc // wc)
         assert threads <= 512 and (br * bk // 8) % threads == 0 and (bc * bk // 8) % threads == 0
-        assert (st - 1) * ((br + bc) * (bk // 8) // threads) <= 63
+        assert b16.vgpr_estimate(br, bc, wr, wc, bk) <= 512 // ((threads // 64 + 3) // 4)
     assert (2, 256, 256, 128, 128, 64) in cfgs
     keys = p16.all_keys()
     assert len(keys) == N_FP16_CONFIGS + N_FP16_SPLITK + 6
@@ -55,13 +59,13 @@ def test_fp16_template_space():
 
 
 def test_fp16_library_names():
-    assert b16.library_for_key((2, 256, 128, 64, 64, 0, 32)).endswith("build/bin_fp16/libgemm_2_256_128_64_64_32.so")
-    assert b16.library_for_key((2, 256, 128, 64, 64, 1, 32)).endswith("build/bin_fp16/libgemm_splitK_2_256_128_64_64_32.so")
+    assert b16.library_for_key((2, 256, 128, 64, 64, 0, 64)).endswith("build/bin_fp16/libgemm_2_256_128_64_64_64.so")
+    assert b16.library_for_key((2, 256, 128, 64, 64, 1, 64)).endswith("build/bin_fp16/libgemm_splitK_2_256_128_64_64_64.so")
     assert b16.library_for_key((0, 1, 128, 0, 0, 0, 0)).endswith("build/bin_fp16/libgemv.so")
     assert b16.library_for_key((0, 16, 128, 0, 0, 1, 0)).endswith("build/bin_fp16/libgemv_splitK.so")
     src, out, defines = b16.compile_job("gemm_splitK", 2, 128, 64, 64, 32, 64)
     assert src.endswith("src_template/MI355X_FP16/gemm.hip")
-    assert defines == {"SPLIT_K": 8, "LDS_STAGES": 2, "BLOCK_ROWS": 128, "BLOCK_COLS": 64, "WAVE_ROWS": 64,
+    assert defines == {"SPLIT_K": 8, "K_STAGES": 2, "BLOCK_ROWS": 128, "BLOCK_COLS": 64, "WAVE_ROWS": 64,
                        "WAVE_COLS": 32, "BLOCK_K": 64}
     cmd = helix_runtime.compile_command(src, out, defines)
     assert "--offload-arch=gfx950" in cmd and "-DBLOCK_ROWS=128" in cmd and "-shared" in cmd
@@ -244,10 +248,10 @@ def test_missing_library_fails_loudly(tmp_path):
 
 
 def test_info_matches_file_name():
-    path = b16.kernel_library("gemm", 2, 256, 128, 64, 64, 32)
+    path = b16.kernel_library("gemm", 2, 256, 128, 64, 64, 64)
     if not os.path.exists(path):
         pytest.skip("kernel libraries are not built")
     info = hip_ctypes.HelixLib(path).info()
-    assert (info["lds_stages"], info["block_rows"], info["block_cols"], info["wave_rows"], info["wave_cols"],
-            info["block_k"], info["split_k"]) == (2, 256, 128, 64, 64, 32, 1)
-    assert info["threads"] == 64 * 4 * 2 and info["lds_bytes"] == 2 * (256 + 128) * 32 * 2
+    assert (info["k_stages"], info["block_rows"], info["block_cols"], info["wave_rows"], info["wave_cols"],
+            info["block_k"], info["split_k"]) == (2, 256, 128, 64, 64, 64, 1)
+    assert info["threads"] == 64 * 4 * 2 and info["lds_bytes"] == 2 * (256 + 128) * 64 * 2
