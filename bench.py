@@ -88,6 +88,10 @@ def main():
     ap.add_argument("--no-gemv", action="store_true")
     ap.add_argument("--kernel-config", type=str, default=None,
                     help="skip the template search and time this configuration, e.g. 2,256,256,64,128,0,64")
+    ap.add_argument("--operands", choices=["seeded", "zeros"], default="seeded",
+                    help="zeros: all-zero operands (no data-dependent power draw; the kernel's structural rate)")
+    ap.add_argument("--torch-matmul", action="store_true",
+                    help="also time torch.matmul (hipBLASLt) on the same operands, reported as torch_matmul_tflops")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 1 GiB device copy (a reference point for HBM traffic counters)")
     args = ap.parse_args()
@@ -119,9 +123,13 @@ def main():
     lib = load(library_for_key(best))
 
     # ---- seeded operands, resident in HBM before the timed region --------------------------------------
-    A_h, B_h = seeded_inputs.gemm_operands(M, N, K, np.float16)          # A (M,K), B (K,N)
-    A = torch.from_numpy(A_h).to(dev)
-    Bt = torch.from_numpy(np.ascontiguousarray(B_h.T)).to(dev)           # device layout: N x K
+    if args.operands == "zeros":
+        A = torch.zeros((M, K), dtype=torch.float16, device=dev)
+        Bt = torch.zeros((N, K), dtype=torch.float16, device=dev)
+    else:
+        A_h, B_h = seeded_inputs.gemm_operands(M, N, K, np.float16)      # A (M,K), B (K,N)
+        A = torch.from_numpy(A_h).to(dev)
+        Bt = torch.from_numpy(np.ascontiguousarray(B_h.T)).to(dev)       # device layout: N x K
     C = torch.empty((M, N), dtype=torch.float16, device=dev)
     wsb = lib.workspace_bytes(M, N, K)
     ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
@@ -164,7 +172,7 @@ def main():
 
     # ---- spot check of the timed result against torch's FP32 matmul on a slice ------------------------------
     ref = A[:256].float() @ Bt[:256].float().t()
-    err = (C[:256, :256].float() - ref).abs().max().item() / ref.abs().max().item()
+    err = (C[:256, :256].float() - ref).abs().max().item() / max(ref.abs().max().item(), 1e-30)
     if not err < 2e-2:
         raise RuntimeError(f"timed GEMM result is wrong: normwise error {err}")
 
@@ -179,6 +187,19 @@ def main():
         "autotune_wall_s": round(autotune_s, 2), "autotune_candidates": tried,
         "roofline": roofline,
     }
+    if args.operands != "seeded":
+        out["config"]["workload"] = f"FP16 GEMM M=N=K={SIZE}, all-zero operands"
+    if args.torch_matmul:
+        # the vendor library on the same operands and layout (A row-major, B stored N x K), wall clock
+        C2 = torch.empty_like(C)
+        for _ in range(args.warmup):
+            torch.matmul(A, Bt.t(), out=C2)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            torch.matmul(A, Bt.t(), out=C2)
+        torch.cuda.synchronize()
+        out["torch_matmul_tflops"] = round(flops / ((time.perf_counter() - t0) / args.steps) / 1e12, 2)
     if not args.no_gemv:
         out["gemv_hbm"] = gemv_rates()
     if not args.no_cpu_baseline:

@@ -46,7 +46,8 @@ def config_cost(k, v, M, N, K):
     splits = split_factor(k, M, N, K)
     num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * splits
     w = math.ceil(num_block / NUM_CU)
-    k_scale = max(K, 64) / PROFILE_K
+    # a tile walks K in whole BLOCK_K steps
+    k_scale = math.ceil(K / k[6]) * k[6] / PROFILE_K
     if k[5] == 1:
         # the profiled value is two rounds of half-K partitions, i.e. about one full-K round; a round of
         # this problem walks K / splits

@@ -13,8 +13,8 @@
 //   BLOCK_ROWS x BLOCK_COLS   workgroup tile of C           (reference BLOCK_ROWS / BLOCK_COLS)
 //   WAVE_ROWS  x WAVE_COLS    tile of C owned by one wave64 (reference WARP_ROWS / WARP_COLS)
 //   BLOCK_K                   K extent of one LDS stage (64 or 128)
-//   K_STAGES                  K tiles in the pipeline: 2 = the tile being multiplied + one staged in
-//                             registers on its way to LDS, 3 = two staged      (reference K_STAGE)
+//   K_STAGES                  K tiles in the pipeline beside the one being loaded: the tile being multiplied
+//                             and the one on its way to LDS; 2 is the only depth    (reference K_STAGE)
 //   SPLIT_K                   1: each workgroup walks all of K.  > 1: K is partitioned over blockIdx.y into
 //                             2 .. SPLIT_K ranges, as many as it takes to give every compute unit a
 //                             workgroup (FP32 workspace + fixed-order reduction kernel)
@@ -25,7 +25,7 @@
 //     chip runs against its power limit, MFMA-only loops measure 1.95 PFLOP/s with it against 1.69.
 //   * global -> registers (128-bit buffer loads; hardware bounds checking zero-fills rows beyond M / N and
 //     the K tail) -> LDS (ds_write_b128) -> fragments (ds_read_b128).  Two LDS stages; the loads of a tile
-//     are issued one or two tiles ahead and every memory instruction sits behind its own MFMA, evenly
+//     are issued one tile ahead of its LDS writes and every memory instruction sits behind its own MFMA, evenly
 //     spread over the tile, so that the four waves of a workgroup never queue bursts on the CU's single
 //     address unit (a burst of 64 KiB behind a barrier costs more than the k-step it hides in).
 //   * LDS rows are BLOCK_K halves; 16-byte chunk c of row r is stored at chunk (c ^ key(r)), with
@@ -64,7 +64,7 @@
 #define SPLIT_K 1
 #endif
 #ifndef GROUP_ROWS
-#define GROUP_ROWS 8
+#define GROUP_ROWS 4
 #endif
 
 namespace {
@@ -382,9 +382,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     const int ktiles = (k_end - k_begin + BK - 1) / BK;
 
     // Software pipeline over K tiles.  Tile t is multiplied from LDS stage t % 2 while
-    //   * the staging registers that hold tile t+1 (loaded R tiles ago) are written to the other stage with
-    //     ds_write_b128 and each register is refilled with the same slot of tile t+1+R, so a global load has
-    //     R whole K tiles to land;
+    //   * the staging registers that hold tile t+1 (loaded a tile ago) are written to the other stage with
+    //     ds_write_b128 and each register is refilled with the same slot of tile t+2, so a global load has
+    //     a whole K tile to land;
     //   * fragments are read ahead of the MFMAs that use them: the operand with more fragments per k-step
     //     (the "resident" one) is double-buffered by k-step and read one k-step ahead, the other one is
     //     streamed through a small rotating set of registers, PD fragments ahead;
