@@ -4,7 +4,7 @@
  * One shared library == one instantiated kernel template, the way one executable is one
  * instantiated template in the reference (scripts/Ampere_FP16/build_Ampere_FP16.py:7-28 builds
  * `gemm_{K_STAGE}_{BLOCK_ROWS}_{BLOCK_COLS}_{WARP_ROWS}_{WARP_COLS}`; here the same parameters give
- * `libgemm_{LDS_STAGES}_{BLOCK_ROWS}_{BLOCK_COLS}_{WAVE_ROWS}_{WAVE_COLS}.so`).  Every library exports
+ * `libgemm_{K_STAGES}_{BLOCK_ROWS}_{BLOCK_COLS}_{WAVE_ROWS}_{WAVE_COLS}_{BLOCK_K}.so`).  Every library exports
  * every symbol below, so the host side binds one ctypes signature set and swaps libraries per
  * configuration.  An entry point a template does not implement returns HELIX_ERR_UNSUPPORTED.
  *
