@@ -1,7 +1,10 @@
-// MI355X (gfx950 / CDNA4) FP16 GEMV / skinny-GEMM template: no MFMA, HBM-bound weight streaming.
+// MI355X (gfx950 / CDNA4) FP16 GEMV / skinny-GEMM template: HBM-bound weight streaming.
 //
 //   C[M x N] = A[M x K] * B[N x K]^T,  M small (decode batch), B = the weight matrix, streamed once.
-//   FP16 in, FP32 accumulate (v_dot2_f32_f16), FP16 out.
+//   FP16 in, FP32 accumulate, FP16 out.  Up to MFMA_MIN_M - 1 activation rows the products are
+//   v_dot2_f32_f16 with a wave reduction (no MFMA); from MFMA_MIN_M rows on, the vector units would need
+//   more time for the M x K x N dot products than HBM needs for the weights (at M = 16: 48 us against 59 us
+//   for 8192 x 28672, before any overhead), and the same stream feeds v_mfma_f32_16x16x32_f16 instead.
 //
 // Role in the reference: src_template/Ampere_FP16/gemv.cu:152-252 (`mySGemvKernel_Stage4` and its
 // N_TILE dispatch) and gemv_splitK.cu:153-260.  The reference names the streamed matrix A (Mbig x K)
@@ -24,6 +27,18 @@
 //     budget (M_TILE * K * 2 bytes > 64 KiB) or when SPLIT_K asks for it; partials then go to an FP32
 //     workspace and a second kernel sums them in fixed order (deterministic; the reference uses half
 //     atomics, gemv_splitK.cu:213-217).
+//
+// MFMA variant (M >= MFMA_MIN_M)
+//   * a workgroup stages 16 activation rows of its K range (at most 2048 columns) in LDS, rows 16 bytes apart
+//     from a multiple of 256 so that 16 rows of one column sit in 16 different bank groups;
+//   * a wave owns runs of 16 consecutive weight rows; per 256-wide K step it issues eight 16-byte loads per
+//     lane, straight into registers in the operand layout of the MFMA (lane l: row l % 16, columns 8*(l/16)
+//     .. +7 of a 32-wide block): 512 contiguous bytes per row and step, 64 per row and instruction; the same
+//     columns of activation row l % 16 come from LDS;
+//   * eight MFMAs per step accumulate the 16 x 16 block y[m][n]; steps are double-buffered; buffer bounds
+//     checking zero-fills weight rows beyond N;
+//   * K is partitioned over blockIdx.z into ranges of at most 2048 columns, and further until the launch has
+//     enough waves to cover the latency of the stream (FP32 workspace + fixed-order reduce).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -62,6 +77,18 @@
 #ifndef TARGET_WAVES
 #define TARGET_WAVES 2048   // waves a launch aims for: 256 compute units x 8
 #endif
+#ifndef MFMA_MIN_M
+#define MFMA_MIN_M 9        // activation rows from which the MFMA variant takes over (measured crossover)
+#endif
+#ifndef MFMA_TARGET_WAVES
+#define MFMA_TARGET_WAVES 4096
+#endif
+#ifndef MFMA_WAVES_PER_BLOCK
+#define MFMA_WAVES_PER_BLOCK 8
+#endif
+#ifndef MFMA_KCHUNK
+#define MFMA_KCHUNK 1024    // widest K range of a workgroup of the MFMA variant (16 x MFMA_KCHUNK halves of LDS)
+#endif
 
 namespace {
 
@@ -69,6 +96,8 @@ typedef _Float16 half_t;
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half4 __attribute__((ext_vector_type(4)));
 
 constexpr int SPLITK = SPLIT_K;
 constexpr int WPB = WAVES_PER_BLOCK;
@@ -291,6 +320,143 @@ __global__ __launch_bounds__(64 * WPB) void helix_gemv_f16_kernel(const Params p
     }
 }
 
+// ---- MFMA variant -----------------------------------------------------------------------------------------
+constexpr int MSTEP = 256;                      // K extent of one step: eight 16-byte loads per lane, 512 bytes per weight row
+constexpr int MCH = MSTEP / 32;                 // 16-byte chunks per lane and step = MFMAs per step
+constexpr int MFMA_KCHUNK_MAX = MFMA_KCHUNK;     // K range of a workgroup: 16 staged activation rows of this width
+constexpr int MWPB = MFMA_WAVES_PER_BLOCK;
+constexpr int XROW_PAD = 16;                    // bytes between staged rows: 16 rows of one column hit 16 bank groups
+
+#ifndef MFMA_LOAD_AUX
+#define MFMA_LOAD_AUX 0   // cache policy bits of the weight loads (non-temporal, 2, measures 5-10 % slower: the two
+                          // halves of a 128-byte line are fetched by consecutive instructions)
+#endif
+__device__ __forceinline__ half8 buf_load8(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, MFMA_LOAD_AUX));
+}
+
+__global__ __launch_bounds__(64 * MWPB) void helix_gemv_f16_mfma_kernel(const Params p) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, q = lane >> 4;
+    const int m0 = blockIdx.y * 16;
+    const int kchunk = p.kchunk;                                    // multiple of MSTEP
+    const int k_begin = (int)blockIdx.z * kchunk;
+    const int k_end = (k_begin + kchunk) < p.K ? (k_begin + kchunk) : p.K;
+    const int xrow = kchunk * 2 + XROW_PAD;                          // bytes per staged activation row
+
+    const int ngroups = (p.N + 15) / 16;
+    const int group_first = (blockIdx.x * MWPB + wave) * p.rows_per_wave;      // in units of 16-row groups
+    const int group_last = (group_first + p.rows_per_wave) < ngroups ? (group_first + p.rows_per_wave) : ngroups;
+
+    // weights of 16-row group g: load c of a step reads, in lane (r, q), columns 32*c + 8*q .. +7 of row r -- one
+    // instruction covers 64 contiguous bytes of each of 16 rows, the eight loads of a step 512 contiguous bytes
+    // per row.  Rows beyond N read as zeros (buffer bounds).
+    auto w_rsrc = [&](int g) -> __amdgpu_buffer_rsrc_t {
+        const int n0 = g * 16;
+        const int rows_w = (p.N - n0) < 16 ? (p.N - n0) : 16;
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(p.B + (size_t)n0 * p.ldb), 0,
+                                                 (int)(((size_t)(rows_w - 1) * p.ldb + p.K) * 2), 0x00020000);
+    };
+    const int woff = (r * p.ldb + 8 * q) * 2;
+    auto load_step = [&](half8 (&w)[MCH], __amdgpu_buffer_rsrc_t rw, int k) {
+#pragma unroll
+        for (int c = 0; c < MCH; c++) w[c] = buf_load8(rw, woff + c * 64, k * 2);
+    };
+    auto load_step_tail = [&](half8 (&w)[MCH], __amdgpu_buffer_rsrc_t rw, int k) {
+#pragma unroll
+        for (int c = 0; c < MCH; c++) w[c] = buf_load8(rw, (k + 32 * c + 8 * q < k_end) ? woff + c * 64 : 0x7fffffff, k * 2);
+    };
+
+    // the first step of the first group is requested before the activations are staged
+    half8 wa[MCH], wb[MCH];
+    __amdgpu_buffer_rsrc_t rw = w_rsrc(group_first < ngroups ? group_first : 0);
+    const bool full_first = (k_begin + MSTEP <= k_end);
+    if (group_first < group_last) {
+        if (full_first) load_step(wa, rw, k_begin); else load_step_tail(wa, rw, k_begin);
+    }
+
+    // ---- stage the activations: 16 rows x kchunk, zero beyond M and beyond the K range --------------------
+    {
+        const int chunks_per_row = kchunk / 8;
+        const int total = 16 * chunks_per_row;
+        for (int c = tid; c < total; c += 64 * MWPB) {
+            const int m = c / chunks_per_row, kc = (c % chunks_per_row) * 8;
+            intx4 v = {0, 0, 0, 0};
+            if (m0 + m < p.M && k_begin + kc < k_end) v = *(const intx4*)(p.A + (size_t)(m0 + m) * p.lda + k_begin + kc);
+            *(intx4*)(smem + m * xrow + kc * 2) = v;
+        }
+    }
+    __syncthreads();
+    const unsigned char* xl = smem + r * xrow + 8 * q * 2;           // this lane's activation row and column base
+
+    for (int g = group_first; g < group_last; g++) {
+        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
+        auto mfma_step = [&](const half8 (&w)[MCH], int k) {
+#pragma unroll
+            for (int c = 0; c < MCH; c++) {
+                const half8 xv = *(const half8*)(xl + (k - k_begin) * 2 + c * 64);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[c], xv, acc, 0, 0, 0);
+            }
+        };
+        // double-buffered steps: step s+1 is requested before the MFMAs of step s; wa holds the step at k
+        int k = k_begin;
+        for (; k + 3 * MSTEP <= k_end; k += 2 * MSTEP) {
+            load_step(wb, rw, k + MSTEP);
+            mfma_step(wa, k);
+            load_step(wa, rw, k + 2 * MSTEP);
+            mfma_step(wb, k + MSTEP);
+        }
+        // at most two steps and a partial one are left; wa holds the step at k
+        bool have_b = false;
+        if (k + MSTEP < k_end) {
+            if (k + 2 * MSTEP <= k_end) load_step(wb, rw, k + MSTEP); else load_step_tail(wb, rw, k + MSTEP);
+            have_b = true;
+        }
+        mfma_step(wa, k);
+        k += MSTEP;
+        if (have_b) {
+            if (k + MSTEP < k_end) {          // a third, partial step behind wb
+                load_step_tail(wa, rw, k + MSTEP);
+                mfma_step(wb, k);
+                mfma_step(wa, k + MSTEP);
+            } else {
+                mfma_step(wb, k);
+            }
+        }
+        // request the next group's first step, then store this group underneath it
+        if (g + 1 < group_last) {
+            rw = w_rsrc(g + 1);
+            if (full_first) load_step(wa, rw, k_begin); else load_step_tail(wa, rw, k_begin);
+        }
+
+        // lane l holds y[m0 + l % 16][n0 + 4*(l/16) + {0..3}]
+        const int m = m0 + r, n = g * 16 + 4 * q;
+        if (m < p.M && n < p.N) {
+            if (p.ksplit > 1) {
+                float* dst = p.ws + ((size_t)blockIdx.z * p.M + m) * p.N + n;
+                if ((p.N & 3) == 0) *(floatx4*)dst = acc;
+                else
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < p.N) dst[e] = acc[e];
+            } else {
+                half_t* dst = p.C + (size_t)m * p.ldc + n;
+                if ((p.ldc & 3) == 0 && (((uintptr_t)p.C) & 7) == 0 && n + 4 <= p.N) {
+                    half4 h = {(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
+                    *(half4*)dst = h;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (n + e < p.N) dst[e] = (half_t)acc[e];
+                }
+            }
+        }
+    }
+}
+
 __global__ void helix_gemv_splitk_reduce_kernel(const float* ws, half_t* C, int M, int N, int ldc, int splits) {
     const size_t total = (size_t)M * N;
     for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
@@ -310,17 +476,17 @@ namespace tpl {
 constexpr int kElemBytes = 2;
 
 inline const char* info_json() {
-    static char buf[768];
+    static char buf[1024];
     static bool done = false;
     if (!done) {
         snprintf(buf, sizeof(buf),
-                 "{\"family\": \"gemv_f16\", \"arch\": \"gfx950\", \"mfma\": \"none\", \"lds_stages\": 0, "
+                 "{\"family\": \"gemv_f16\", \"arch\": \"gfx950\", \"mfma\": \"none below %d activation rows, v_mfma_f32_16x16x32_f16 from there\", \"lds_stages\": 0, "
                  "\"block_rows\": 1, \"block_cols\": 128, \"wave_rows\": 0, \"wave_cols\": 0, \"split_k\": %d, "
                  "\"threads\": %d, \"lds_bytes\": %d, \"k_step\": %d, "
                  "\"layout_a\": \"M x K row-major f16 (activations)\", "
                  "\"layout_b\": \"N x K row-major f16 (streamed weights)\", \"layout_c\": \"M x N row-major f16\", "
                  "\"accumulate\": \"f32\", \"k_multiple\": 8, \"ld_multiple\": 8}",
-                 SPLITK, 64 * WPB, X_LDS_BYTES, KSTEP);
+                 MFMA_MIN_M, SPLITK, 64 * WPB, X_LDS_BYTES, KSTEP);
         done = true;
     }
     return buf;
@@ -329,7 +495,25 @@ inline const char* info_json() {
 constexpr int mtile_of(int M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
 // K partitioning: enough ranges that M_TILE activation rows of one range fit X_LDS_BYTES, at least SPLIT_K
-inline void k_partition(int M, int K, int* kchunk, int* ksplit) {
+// MFMA variant: K ranges are multiples of 256 and at most 2048 wide (the staged activations), at least 512
+// wide, as many as bring the launch to about MFMA_TARGET_WAVES waves of 16 weight rows each, at least SPLIT_K
+inline void k_partition_mfma(int N, int K, int* kchunk, int* ksplit) {
+    const int steps = (K + MSTEP - 1) / MSTEP;
+    const long long groups = (N + 15) / 16;
+    long long split = (MFMA_TARGET_WAVES + groups - 1) / groups;
+    const long long max_split = steps / 2 > 1 ? steps / 2 : 1;
+    if (split > max_split) split = max_split;
+    const long long min_split = (steps + MFMA_KCHUNK_MAX / MSTEP - 1) / (MFMA_KCHUNK_MAX / MSTEP);
+    if (split < min_split) split = min_split;
+    if (split < SPLITK) split = SPLITK;
+    if (split > steps) split = steps;
+    const int per = (int)((steps + split - 1) / split);
+    *kchunk = per * MSTEP;
+    *ksplit = (steps + per - 1) / per;
+}
+
+inline void k_partition(int M, int N, int K, int* kchunk, int* ksplit) {
+    if (M >= MFMA_MIN_M) return k_partition_mfma(N, K, kchunk, ksplit);
     const int mt = mtile_of(M);
     const int steps = (K + KSTEP - 1) / KSTEP;
     int max_steps = X_LDS_BYTES / (mt * KSTEP * 2);
@@ -344,7 +528,7 @@ inline void k_partition(int M, int K, int* kchunk, int* ksplit) {
 
 inline size_t workspace_bytes(int M, int N, int K) {
     int kchunk, ksplit;
-    k_partition(M, K, &kchunk, &ksplit);
+    k_partition(M, N, K, &kchunk, &ksplit);
     return ksplit > 1 ? (size_t)ksplit * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
@@ -369,6 +553,24 @@ inline int launch_cfg(Params p, hipStream_t s) {
     return (int)hipGetLastError();
 }
 
+inline int launch_mfma(Params p, hipStream_t s) {
+    if ((long long)16 * p.ldb * 2 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    const long long groups = (p.N + 15) / 16;
+    // 16-row groups per wave: as many as keep the launch near MFMA_TARGET_WAVES waves (the staged activations
+    // are shared by all groups a workgroup walks)
+    long long gpw = (groups * p.ksplit + MFMA_TARGET_WAVES - 1) / MFMA_TARGET_WAVES;
+    if (gpw < 1) gpw = 1;
+    p.rows_per_wave = (int)gpw;
+    const long long waves = (groups + gpw - 1) / gpw;
+    const int lds = 16 * (p.kchunk * 2 + XROW_PAD);
+    static int attr_rc = (int)hipFuncSetAttribute((const void*)helix_gemv_f16_mfma_kernel,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr_rc) return attr_rc;
+    dim3 grid((unsigned)((waves + MWPB - 1) / MWPB), (p.M + 15) / 16, p.ksplit), block(64 * MWPB);
+    hipLaunchKernelGGL(helix_gemv_f16_mfma_kernel, grid, block, lds, s, p);
+    return (int)hipGetLastError();
+}
+
 inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc, void* ws,
                 size_t ws_bytes, hipStream_t s) {
     if (K % 8 != 0 || lda % 8 != 0 || ldb % 8 != 0) return HELIX_ERR_INVALID_VALUE;
@@ -376,7 +578,7 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)C & 1)) return HELIX_ERR_INVALID_VALUE;
     if ((M + 15) / 16 > 65535) return HELIX_ERR_INVALID_VALUE;
     Params p{(const half_t*)A, (const half_t*)B, (half_t*)C, (float*)ws, M, N, K, lda, ldb, ldc, 0, 1, 1};
-    k_partition(M, K, &p.kchunk, &p.ksplit);
+    k_partition(M, N, K, &p.kchunk, &p.ksplit);
     if (p.ksplit > 65535) return HELIX_ERR_INVALID_VALUE;
     if (p.ksplit > 1) {
         if (!ws || ws_bytes < workspace_bytes(M, N, K)) return HELIX_ERR_WORKSPACE;
@@ -384,7 +586,8 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     int rc;
     // activation-row tile, like the reference's N_TILE pick from the skinny extent (gemv.cu:232-250); wider
     // tiles take more weight rows per pass so that one LDS read of the activations feeds several rows
-    switch (mtile_of(M)) {
+    if (M >= MFMA_MIN_M) rc = launch_mfma(p, s);
+    else switch (mtile_of(M)) {
         case 1: rc = launch_cfg<1, GEMV_R1, GEMV_KU1>(p, s); break;
         case 2: rc = launch_cfg<2, GEMV_R2, GEMV_KU2>(p, s); break;
         case 4: rc = launch_cfg<4, GEMV_R4, GEMV_KU4>(p, s); break;

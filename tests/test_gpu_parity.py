@@ -201,7 +201,7 @@ def test_gemm_f16_rejects_bad_arguments():
 @pytest.mark.parametrize("name", ["gemv", "gemv_splitK"])
 def test_gemv_f16_vs_oracle(name):
     lib = load(b16.kernel_library(name))
-    for M in (1, 2, 3, 4, 5, 8, 16, 17):
+    for M in (1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 33):
         for (N, K) in [(128, 512), (1000, 1032), (4096, 4096), (9001, 520), (20000, 8)]:
             x, W = seeded_inputs.gemv_operands(M, N, K)
             got = run_gemm_f16(lib, x, W)
@@ -214,7 +214,7 @@ def test_gemv_f16_integer_inputs_exact():
     rng = np.random.default_rng(6)
     for name in ("gemv", "gemv_splitK"):
         lib = load(b16.kernel_library(name))
-        for (M, N, K) in [(1, 777, 1536), (4, 2050, 520), (16, 300, 1024), (7, 4100, 2056)]:
+        for (M, N, K) in [(1, 777, 1536), (4, 2050, 520), (16, 300, 1024), (7, 4100, 2056), (11, 1030, 776), (35, 257, 264)]:
             x = rng.integers(-2, 3, (M, K)).astype(np.float16)
             W = rng.integers(-1, 2, (K, N)).astype(np.float16)
             want = x.astype(np.int64) @ W.astype(np.int64)
