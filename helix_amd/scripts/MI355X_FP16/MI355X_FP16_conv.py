@@ -3,8 +3,9 @@
 Mirrors scripts/Ampere_FP16/Ampere_FP16_conv.py:420-446: the conv is mapped to GEMM extents
 M = batch*OH*OW, N = OC, K = IC*kH*kW (:432-434), the GEMM cost model picks the configuration, and
 the cost is measured.  The reference runs an im2col executable plus the GEMM executable and adds the
-two times (:437-445); here the selected configuration's library gathers the A tile on the fly, so
-there is one kernel and one time.
+two times (:437-445); here the selected configuration's library gathers the A tile on the fly (one
+kernel, one time) when IC is a multiple of 8, and runs im2col + weight repack + GEMM on one stream
+inside the same entry point otherwise (one time for the three kernels).
 """
 import math
 import os

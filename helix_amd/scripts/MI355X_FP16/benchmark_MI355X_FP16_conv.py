@@ -15,9 +15,6 @@ def MI355X_FP16_Helix_op_level_Conv_benchmark(backend="hip"):
 
     shape_list = get_conv_op_shape_list()
     for batch, input_channel, H, W, output_channel, kH, kW, stride, pad in shape_list:
-        if input_channel % 8 != 0:
-            print(f'Helix: skipped (IC={input_channel} needs the explicit im2col path)')
-            continue
         _, helix_tflops = get_MI355X_FP16_conv_Helix_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, backend)
         print(f'Helix: {helix_tflops:.2f} TFLOPS')
 

@@ -13,8 +13,6 @@ root_path = os.getcwd()
 def _summed_cost(prof_dict, shape_list, backend):
     total = 0
     for batch, input_channel, H, W, output_channel, kH, kW, stride, pad in shape_list:
-        if input_channel % 8 != 0:
-            continue   # first layers (IC=3) need the explicit im2col path, which this backend does not have yet
         cost, _ = get_MI355X_FP16_conv_Helix_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, backend)
         total += cost
     return total

@@ -1,6 +1,7 @@
 """Convolution runner of the MI355X_FP32 backend (implicit GEMM, NHWC, FP32).
-Mirrors scripts/Ampere_FP32/Ampere_FP32_conv.py:89-110; one kernel instead of im2col + SGEMM (the
-reference even borrows the FP16 im2col binary here, :107)."""
+Mirrors scripts/Ampere_FP32/Ampere_FP32_conv.py:89-110; one kernel instead of im2col + SGEMM when IC is
+a multiple of 4 (the reference even borrows the FP16 im2col binary here, :107), FP32 im2col + SGEMM
+inside the same entry point otherwise."""
 import math
 import os
 

@@ -17,6 +17,7 @@ HELIX_ERR_WORKSPACE = 2001
 ABI_SYMBOLS = (
     "helix_info",
     "helix_workspace_bytes",
+    "helix_conv_workspace_bytes",
     "helix_gemm",
     "helix_conv2d",
     "helix_gemm_timed",
@@ -48,6 +49,8 @@ class HelixLib:
         L.helix_info.restype = _i
         L.helix_workspace_bytes.argtypes = [_i, _i, _i]
         L.helix_workspace_bytes.restype = _sz
+        L.helix_conv_workspace_bytes.argtypes = [_i] * 9
+        L.helix_conv_workspace_bytes.restype = _sz
         L.helix_gemm.argtypes = [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]
         L.helix_gemm.restype = _i
         L.helix_conv2d.argtypes = [_vp, _vp, _vp] + [_i] * 9 + [_vp, _sz, _vp]
@@ -74,6 +77,9 @@ class HelixLib:
 
     def workspace_bytes(self, M, N, K):
         return int(self._lib.helix_workspace_bytes(M, N, K))
+
+    def conv_workspace_bytes(self, batch, H, W, IC, OC, kH, kW, stride, pad):
+        return int(self._lib.helix_conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad))
 
     # -- launches (raw device pointers as ints) -------------------------------------------------------
     def gemm(self, A, B, C, M, N, K, lda, ldb, ldc, ws=0, ws_bytes=0, stream=0, check=True):

@@ -41,6 +41,7 @@
 #include <type_traits>
 
 #include "helix_abi.h"
+#include "helix_im2col.h"
 
 #ifndef BLOCK_ROWS
 #define BLOCK_ROWS 256
@@ -609,7 +610,7 @@ inline const char* info_json() {
                  "\"block_k\": %d, \"split_k\": %d, \"threads\": %d, \"lds_bytes\": %d, "
                  "\"layout_a\": \"M x K row-major f16\", \"layout_b\": \"N x K row-major f16\", "
                  "\"layout_c\": \"M x N row-major f16\", \"accumulate\": \"f32\", "
-                 "\"k_multiple\": 8, \"ld_multiple\": 8, \"conv\": \"NHWC x [OC][kH][kW][IC], IC %% 8 == 0\"}",
+                 "\"k_multiple\": 8, \"ld_multiple\": 8, \"conv\": \"NHWC x [OC][kH][kW][IC]; implicit GEMM when IC %% 8 == 0, else column buffer in the workspace\"}",
                  STAGES, BM, BN, WM, WN, BK, SPLITK, NTHREADS, LDS_BYTES);
         done = true;
     }
@@ -688,15 +689,52 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     return launch<0>(p, ws, ws_bytes, s);
 }
 
+// Convolutions whose channel count is not a multiple of 8 go through a column buffer (K padded to a multiple
+// of 8) and repacked weights in the workspace, then through the GEMM above.
+inline int conv_padded_k(int IC, int kH, int kW) { return (IC * kH * kW + 7) / 8 * 8; }
+
+inline size_t conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad) {
+    const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
+    const long long M = (long long)batch * OH * OW;
+    if (M > 0x7fffffffLL) return 0;
+    if (IC % 8 == 0) return workspace_bytes((int)M, OC, IC * kH * kW);
+    const int Kp = conv_padded_k(IC, kH, kW);
+    return helix_im2col::align256((size_t)M * Kp * 2) + helix_im2col::align256((size_t)OC * Kp * 2) +
+           workspace_bytes((int)M, OC, Kp);
+}
+
+inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
+                           int kW, int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
+    const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
+    const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
+    if (M > 0x7fffffffLL || K > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    const int Kp = conv_padded_k(IC, kH, kW);
+    const size_t col_bytes = helix_im2col::align256((size_t)M * Kp * 2);
+    const size_t wp_bytes = helix_im2col::align256((size_t)OC * Kp * 2);
+    if (!ws || ws_bytes < conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad)) return HELIX_ERR_WORKSPACE;
+    half_t* col = (half_t*)ws;
+    half_t* wp = (half_t*)((unsigned char*)ws + col_bytes);
+    void* rest = (unsigned char*)ws + col_bytes + wp_bytes;
+    const helix_im2col::Geom g{H, W, IC, OH, OW, kW, stride, pad, (int)M, (int)K};
+    hipLaunchKernelGGL((helix_im2col::im2col_rows_kernel<half_t, 8>), dim3(helix_im2col::grid_for((size_t)M * (Kp / 8))),
+                       dim3(256), 0, s, (const half_t*)x, col, g, Kp);
+    hipLaunchKernelGGL((helix_im2col::pack_weights_rows_kernel<half_t>), dim3(helix_im2col::grid_for((size_t)OC * Kp)),
+                       dim3(256), 0, s, (const half_t*)w, wp, OC, (int)K, Kp);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return gemm(col, wp, y, (int)M, OC, Kp, Kp, Kp, OC, rest, ws_bytes - col_bytes - wp_bytes, s);
+}
+
 inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
                   int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
-    if (IC % 8 != 0) return HELIX_ERR_INVALID_VALUE;  // a 16-byte chunk must stay inside one filter tap
+    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 1)) return HELIX_ERR_INVALID_VALUE;
+    if (IC % 8 != 0)   // a 16-byte chunk of the implicit gather must stay inside one filter tap
+        return conv2d_explicit(x, w, y, batch, H, W, IC, OC, kH, kW, stride, pad, ws, ws_bytes, s);
     const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
     const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
     const long long xbytes = (long long)batch * H * W * IC * 2;
     if (M > 0x7fffffffLL || K > 0x7fffffffLL || xbytes >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
     if ((long long)BN * K * 2 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
-    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 1)) return HELIX_ERR_INVALID_VALUE;
     Params p{};
     p.A = (const half_t*)x; p.B = (const half_t*)w; p.C = (half_t*)y; p.ws = (float*)ws;
     p.M = (int)M; p.N = OC; p.K = (int)K; p.lda = 0; p.ldb = (int)K; p.ldc = OC;

@@ -606,6 +606,8 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     return 0;
 }
 
+inline size_t conv_workspace_bytes(int, int, int, int, int, int, int, int, int) { return 0; }
+
 inline int conv2d(const void*, const void*, void*, int, int, int, int, int, int, int, int, int, void*, size_t,
                   hipStream_t) {
     return HELIX_ERR_UNSUPPORTED;

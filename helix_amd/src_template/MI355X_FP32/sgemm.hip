@@ -20,6 +20,7 @@
 #include <stdint.h>
 
 #include "helix_abi.h"
+#include "helix_im2col.h"
 
 #ifndef BM
 #define BM 128
@@ -287,7 +288,7 @@ inline const char* info_json() {
                  "\"block_k\": %d, \"split_k\": 1, \"threads\": %d, \"lds_bytes\": %d, "
                  "\"layout_a\": \"K x M row-major f32 (A transposed)\", \"layout_b\": \"K x N row-major f32\", "
                  "\"layout_c\": \"M x N row-major f32\", \"accumulate\": \"f32\", "
-                 "\"k_multiple\": 1, \"ld_multiple\": 4, \"conv\": \"NHWC x [OC][kH][kW][IC], IC %% 4 == 0\"}",
+                 "\"k_multiple\": 1, \"ld_multiple\": 4, \"conv\": \"NHWC x [OC][kH][kW][IC]; implicit GEMM when IC %% 4 == 0, else column buffer in the workspace\"}",
                  BM, BN, WAVE_M, WAVE_N, BK, NTHREADS, LDS_BYTES);
         done = true;
     }
@@ -330,15 +331,46 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     return launch<false>(p, s);
 }
 
+// Convolutions whose channel count is not a multiple of 4 go through a column buffer (K x M, the A layout of
+// this template) and transposed weights (K x N) in the workspace, then through the GEMM above.
+inline size_t conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad) {
+    if (IC % 4 == 0) return 0;
+    const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
+    const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
+    const long long Mp = (M + 3) / 4 * 4, Np = (OC + 3) / 4 * 4;
+    return helix_im2col::align256((size_t)K * Mp * 4) + helix_im2col::align256((size_t)K * Np * 4);
+}
+
+inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
+                           int kW, int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
+    const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
+    const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
+    if (M > 0x7fffffffLL - 4 || K > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    const int Mp = (int)((M + 3) / 4 * 4), Np = (OC + 3) / 4 * 4;
+    const size_t col_bytes = helix_im2col::align256((size_t)K * Mp * 4);
+    if (!ws || ws_bytes < conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad)) return HELIX_ERR_WORKSPACE;
+    float* col = (float*)ws;
+    float* wt = (float*)((unsigned char*)ws + col_bytes);
+    const helix_im2col::Geom g{H, W, IC, OH, OW, kW, stride, pad, (int)M, (int)K};
+    hipLaunchKernelGGL((helix_im2col::im2col_cols_kernel<float>), dim3(helix_im2col::grid_for((size_t)K * Mp)), dim3(256),
+                       0, s, (const float*)x, col, g, Mp);
+    hipLaunchKernelGGL((helix_im2col::pack_weights_cols_kernel<float>), dim3(helix_im2col::grid_for((size_t)K * Np)),
+                       dim3(256), 0, s, (const float*)w, wt, OC, (int)K, Np);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return gemm(col, wt, y, (int)M, OC, (int)K, Mp, Np, OC, nullptr, 0, s);
+}
+
 inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
-                  int stride, int pad, void*, size_t, hipStream_t s) {
-    if (IC % 4 != 0) return HELIX_ERR_INVALID_VALUE;  // a 16-byte chunk must stay inside one filter tap
+                  int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
+    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 3)) return HELIX_ERR_INVALID_VALUE;
+    if (IC % 4 != 0)   // a 16-byte chunk of the implicit gather must stay inside one filter tap
+        return conv2d_explicit(x, w, y, batch, H, W, IC, OC, kH, kW, stride, pad, ws, ws_bytes, s);
     const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
     const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
     const long long xbytes = (long long)batch * H * W * IC * 4;
     if (M > 0x7fffffffLL || K > 0x7fffffffLL || xbytes >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
     if ((long long)BN * K * 4 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
-    if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 3)) return HELIX_ERR_INVALID_VALUE;
     Params p{};
     p.A = (const float*)x; p.B = (const float*)w; p.C = (float*)y;
     p.M = (int)M; p.N = OC; p.K = (int)K; p.lda = 0; p.ldb = (int)K; p.ldc = OC;

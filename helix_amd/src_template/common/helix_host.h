@@ -6,6 +6,7 @@
 //     constexpr int kElemBytes;                       // 2 (FP16) or 4 (FP32)
 //     const char* info_json();
 //     size_t workspace_bytes(int M, int N, int K);
+//     size_t conv_workspace_bytes(int B, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad);
 //     int gemm(const void*, const void*, void*, int M, int N, int K, int lda, int ldb, int ldc,
 //              void* ws, size_t ws_bytes, hipStream_t);
 //     int conv2d(const void*, const void*, void*, int B, int H, int W, int IC, int OC, int kH, int kW,
@@ -130,6 +131,12 @@ size_t helix_workspace_bytes(int M, int N, int K) {
     return tpl::workspace_bytes(M, N, K);
 }
 
+size_t helix_conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad) {
+    if (batch <= 0 || H <= 0 || W <= 0 || IC <= 0 || OC <= 0 || kH <= 0 || kW <= 0 || stride <= 0 || pad < 0) return 0;
+    if (H + 2 * pad < kH || W + 2 * pad < kW) return 0;
+    return tpl::conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad);
+}
+
 int helix_gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
                void* workspace, size_t workspace_bytes, void* stream) {
     if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return HELIX_ERR_INVALID_VALUE;
@@ -226,7 +233,7 @@ int helix_bench_conv(int batch, int IC, int H, int W, int OC, int kH, int kW, in
     if ((rc = bufs.alloc(&x, xe * eb))) return rc;
     if ((rc = bufs.alloc(&w, we * eb))) return rc;
     if ((rc = bufs.alloc(&y, ye * eb))) return rc;
-    size_t wsb = tpl::workspace_bytes(batch * OH * OW, OC, IC * kH * kW);
+    size_t wsb = tpl::conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad);
     if ((rc = bufs.alloc(&ws, wsb))) return rc;
     if ((rc = helix_host::fill(x, xe, eb, 0.5f, 1u, nullptr))) return rc;
     if ((rc = helix_host::fill(w, we, eb, 0.5f, 2u, nullptr))) return rc;

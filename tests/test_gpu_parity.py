@@ -258,8 +258,10 @@ def run_conv(lib, x, w, stride, pad, dtype):
     OH, OW = O.conv_out_hw(H, W, kH, kW, stride, pad)
     dx, dw = dev(x), dev(w)
     dy = torch.full((batch, OH, OW, OC), float("nan"), dtype=dtype, device="cuda:0")
-    lib.conv2d(dx.data_ptr(), dw.data_ptr(), dy.data_ptr(), batch, H, W, IC, OC, kH, kW, stride, pad, 0, 0,
-               torch.cuda.current_stream().cuda_stream)
+    wsb = lib.conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad)
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda:0")
+    lib.conv2d(dx.data_ptr(), dw.data_ptr(), dy.data_ptr(), batch, H, W, IC, OC, kH, kW, stride, pad,
+               ws.data_ptr() if wsb else 0, wsb, torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     return dy.cpu().numpy()
 
@@ -267,13 +269,16 @@ def run_conv(lib, x, w, stride, pad, dtype):
 CONV_GEOMS = [(2, 14, 14, 16, 24, 3, 3, 1, 1), (2, 15, 13, 8, 8, 3, 3, 2, 1), (3, 8, 8, 32, 16, 1, 1, 2, 0),
               (1, 12, 12, 8, 40, 5, 5, 1, 2), (2, 9, 9, 64, 64, 3, 3, 1, 1), (1, 7, 7, 24, 16, 3, 3, 1, 0),
               (2, 6, 10, 72, 8, 1, 1, 1, 0)]
+# channel counts that are not a multiple of the gather chunk: explicit im2col + GEMM through the workspace
+CONV_GEOMS_ODD = [(2, 20, 20, 3, 16, 7, 7, 2, 3), (1, 9, 11, 1, 8, 5, 5, 2, 0), (2, 8, 8, 25, 24, 5, 5, 1, 2),
+                  (1, 10, 10, 6, 10, 3, 3, 1, 1), (3, 13, 13, 3, 96, 11, 11, 4, 0)]
 
 
 @pytest.mark.parametrize("cfg", [(2, 128, 128, 64, 64, 64), (2, 64, 64, 32, 32, 64), (2, 256, 64, 64, 32, 64),
                                  (2, 128, 64, 64, 32, 128), (2, 256, 256, 128, 64, 64), (2, 64, 128, 32, 64, 64)])
 def test_conv_f16_vs_oracle(cfg):
     lib = load(b16.kernel_library("gemm", *cfg))
-    for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS:
+    for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS + CONV_GEOMS_ODD:
         x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW)
         got = run_conv(lib, x, w, stride, pad, torch.float16)
         want = O.conv2d_nhwc(x, w, stride, pad)
@@ -299,10 +304,19 @@ def test_conv_f16_golden_and_special_cases():
     wi = rng.integers(-2, 3, (16, 3, 3, 8)).astype(np.float16)
     want = O.conv2d_nhwc(xi.astype(np.float32), wi.astype(np.float32), 2, 1)
     assert np.array_equal(run_conv(lib, xi, wi, 2, 1, torch.float16).astype(np.float32), want)
-    # unsupported channel count is refused, not mis-computed
+    # IC = 3 takes the column-buffer path: exact on integers too, also through a split-K library, and refused
+    # without its workspace rather than mis-computed
+    xi3 = rng.integers(-2, 3, (2, 9, 8, 3)).astype(np.float16)
+    wi3 = rng.integers(-2, 3, (16, 3, 3, 3)).astype(np.float16)
+    want3 = O.conv2d_nhwc(xi3.astype(np.float32), wi3.astype(np.float32), 2, 1)
+    assert np.array_equal(run_conv(lib, xi3, wi3, 2, 1, torch.float16).astype(np.float32), want3)
+    libk = load(b16.kernel_library("gemm_splitK", 2, 64, 64, 32, 32, 64))
+    assert np.array_equal(run_conv(libk, xi3, wi3, 2, 1, torch.float16).astype(np.float32), want3)
+    assert lib.conv_workspace_bytes(1, 8, 8, 3, 8, 3, 3, 1, 1) >= 64 * 32 * 2 + 8 * 32 * 2
+    assert lib.conv_workspace_bytes(1, 8, 8, 8, 8, 3, 3, 1, 1) == 0
     t = torch.zeros(4096, dtype=torch.float16, device="cuda:0")
     assert lib.conv2d(t.data_ptr(), t.data_ptr(), t.data_ptr(), 1, 8, 8, 3, 8, 3, 3, 1, 1, check=False) == \
-        HELIX_ERR_INVALID_VALUE
+        HELIX_ERR_WORKSPACE
 
 
 def test_conv_f16_baseline_layers_sampled():
@@ -385,7 +399,7 @@ def test_sgemm_f32_config1_and_large_k():
 def test_conv_f32_vs_oracle():
     for cfg in [(128, 128, 16, 64, 64), (32, 32, 8, 32, 32), (64, 64, 32, 32, 32)]:
         lib = load(b32.sgemm_library(*cfg))
-        for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS + [(2, 8, 8, 4, 8, 3, 3, 1, 1)]:
+        for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS + CONV_GEOMS_ODD + [(2, 8, 8, 4, 8, 3, 3, 1, 1)]:
             x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW, dtype=np.float32)
             got = run_conv(lib, x, w, stride, pad, torch.float32)
             want = O.conv2d_nhwc(x, w, stride, pad)
