@@ -3,10 +3,21 @@
 Same four entry points and return structure as the reference's
 scripts/utils/get_benchmark_shape_list.py (:1, :17, :29, :38), so the benchmark wrappers iterate them
 the same way.  GEMM shapes are (M, N, K); conv shapes are
-(batch, IC, H, W, OC, kH, kW, stride, pad).  The tables built here are: the transformer projection
-and CNN fully-connected GEMMs of the reference's op-level list, the BERT / LLaMA-2 / GPT-2 op-sets,
-AlexNet, and the five benchmark configurations this backend is measured on (BASELINE_* below).
+(batch, IC, H, W, OC, kH, kW, stride, pad).  The lists are composed in the reference's order from a few
+generators (token counts x projection sizes, graph tables x hidden sizes, batch lists x per-layer
+tables); the long per-layer and DeepBench tables are plain data in benchmark_shapes.json next to this
+file.  The five benchmark configurations this backend is measured on are the BASELINE_* names below.
 """
+import json
+import os
+
+with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "benchmark_shapes.json")) as _f:
+    _TABLES = json.load(_f)
+
+
+def _tuples(name):
+    return [tuple(row) for row in _TABLES[name]]
+
 
 # decode / prefill token counts the reference sweeps: 60 values, mostly primes, from 2 to 1949
 TOKEN_COUNTS = [2, 13, 31, 53, 73, 101, 127, 151, 179, 199, 233, 263, 283, 317, 353, 383, 419, 443, 467, 503, 547,
@@ -27,6 +38,13 @@ CNN_BATCHES = [1, 4, 8, 12, 16, 20, 24, 28, 32, 36, 40, 44, 48, 52, 56, 60, 64]
 
 ALEXNET_LAYERS = [(3, 224, 224, 96, 11, 11, 4, 0), (96, 26, 26, 256, 5, 5, 1, 2), (256, 12, 12, 384, 3, 3, 1, 1),
                   (384, 12, 12, 384, 3, 3, 1, 1), (384, 12, 12, 256, 3, 3, 1, 1)]
+GOOGLENET_LAYERS = _tuples("googlenet_layers")
+VGG_LAYERS = _tuples("vgg_layers")
+RESNET_LAYERS = _tuples("resnet_layers")
+DEEPBENCH_CONV = _tuples("deepbench_conv")
+DEEPBENCH_GEMM = _tuples("deepbench_gemm")
+GNN_GRAPHS = _tuples("gnn_graphs")          # (nodes, input features, classes)
+GNN_HIDDEN = list(_TABLES["gnn_hidden"])
 
 # ---- the five measured configurations ------------------------------------------------------------
 BASELINE_SQUARE_SIZES = [1024, 2048, 4096, 8192]
@@ -42,10 +60,20 @@ BASELINE_BERT_LAYERS = 12
 BASELINE_IRREGULAR_MNK = (4000, 2300, 770)
 
 
+def gnn_MNKList():
+    """Two-layer GCN feature transforms: per hidden size, X[nodes x features] * W1 for every graph, then
+    H[nodes x hidden] * W2 for every graph."""
+    out = []
+    for hidden in GNN_HIDDEN:
+        out += [(nodes, hidden, features) for (nodes, features, _) in GNN_GRAPHS]
+        out += [(nodes, classes, hidden) for (nodes, _, classes) in GNN_GRAPHS]
+    return out
+
+
 def get_gemm_op_MNKList():
     transformer = [(m, n, k) for m in TOKEN_COUNTS for (n, k) in TRANSFORMER_NK]
     cnn_fc = [(m, n, k) for m in CNN_FC_BATCHES for (n, k) in CNN_FC_NK]
-    return transformer + cnn_fc
+    return transformer + cnn_fc + DEEPBENCH_GEMM + gnn_MNKList()
 
 
 def get_llm_opset_MNKList():
@@ -59,16 +87,16 @@ def get_llm_opset_MNKList():
 
 
 def get_conv_op_shape_list():
-    layers = ALEXNET_LAYERS + BASELINE_RESNET50_LAYERS
-    return [(batch,) + shape for batch in CNN_BATCHES for shape in layers]
+    layers = ALEXNET_LAYERS + GOOGLENET_LAYERS + VGG_LAYERS + RESNET_LAYERS
+    return [(batch,) + shape for batch in CNN_BATCHES for shape in layers] + DEEPBENCH_CONV
 
 
 def get_cnn_opset_shape_List():
-    """(AlexNet, ResNet, GoogleNet) per-layer lists.  ResNet here is the six ResNet-50-shaped layers
-    of the measured configuration; the GoogleNet table is not carried yet and is returned empty."""
+    """(AlexNet, ResNet, GoogleNet) per-layer lists over the batch sweep."""
     alexnet = [(batch,) + shape for batch in CNN_BATCHES for shape in ALEXNET_LAYERS]
-    resnet = [(batch,) + shape for batch in CNN_BATCHES for shape in BASELINE_RESNET50_LAYERS]
-    return alexnet, resnet, []
+    resnet = [(batch,) + shape for batch in CNN_BATCHES for shape in RESNET_LAYERS]
+    googlenet = [(batch,) + shape for batch in CNN_BATCHES for shape in GOOGLENET_LAYERS]
+    return alexnet, resnet, googlenet
 
 
 def get_baseline_bert_MNKList():

@@ -164,7 +164,15 @@ def test_prof_dict_roundtrip(tmp_path, monkeypatch):
 
 def test_shape_lists():
     g = shapes.get_gemm_op_MNKList()
-    assert len(g) == 60 * 16 + 8 * 10 and g[0] == (2, 1024, 1024) and g[15] == (2, 4096, 11008)
+    # transformer projections x token counts, CNN fully-connected x batches, DeepBench, two-layer GCNs on 15 graphs
+    assert len(g) == 60 * 16 + 8 * 10 + 84 + 5 * 2 * 15 and g[0] == (2, 1024, 1024) and g[15] == (2, 4096, 11008)
+    assert g[-1] == (1888584, 2, 128) and g[60 * 16 + 8 * 10] == (5124, 700, 2048)
+    assert (2708, 16, 1433) in g and (2708, 7, 16) in g and max(m for (m, _, _) in g) == 1889542
+    conv_all = shapes.get_conv_op_shape_list()
+    assert len(conv_all) == 17 * (5 + 56 + 16 + 20) + 107 and conv_all[0] == (1, 3, 224, 224, 96, 11, 11, 4, 0)
+    alex, res, goog = shapes.get_cnn_opset_shape_List()
+    assert (len(alex), len(res), len(goog)) == (17 * 5, 17 * 20, 17 * 56)
+    assert all(len(s) == 9 and min(s) >= 0 for s in conv_all)
     bert, llama, gpt2 = shapes.get_llm_opset_MNKList()
     assert len(bert) == 60 * 73 and len(llama) == 60 * 4 and len(gpt2) == 60 * 96
     bb = shapes.get_baseline_bert_MNKList()
