@@ -9,7 +9,7 @@ import os
 
 from utils.helix_runtime import load
 from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
-from MI355X_FP16.build_MI355X_FP16 import library_for_key, SPLITK_MAX
+from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, SPLITK_MAX
 from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K
 
 root_path = os.getcwd()
@@ -96,6 +96,15 @@ def get_MI355X_FP16_gemm_Helix_result(prof_dict, M, N, K, backend="hip"):
     tflops = 2 * M * N * K / 1e9 / cost
 
     return cost, tflops
+
+
+def get_MI355X_FP16_gemm_rocblas_result(M, N, K):
+    """The vendor library on the same problem (rocblas_gemm_ex, FP16 in / FP32 compute), timed the same way.
+    Mirrors get_Ampere_FP16_gemm_cublas_result (Ampere_FP16_gemm.py:548-553)."""
+    lib = load(kernel_library("rocblas_f16"))
+    _, avg, _ = lib.bench(M, N, K, warmup=10, iters=10, outer=1, rotate_bytes=0)
+    cost = avg * 1e3
+    return cost, 2 * M * N * K / 1e9 / cost
 
 
 def get_MI355X_FP16_gemm_Oracle_result(prof_dict, M, N, K):

@@ -141,7 +141,22 @@ def build_jobs():
             jobs.append(compile_job("gemm_splitK", *cfg))
     jobs.append(compile_job("gemv"))
     jobs.append(compile_job("gemv_splitK"))
+    jobs.append(rocblas_job())
     return jobs
+
+
+def rocblas_job():
+    """The vendor comparator, like the reference's `compile_kernel("cublas_f16")` (build_Ampere_FP16.py:72-76)."""
+    return (f"{SRC_ROOT}/MI355X_FP16/rocblas_f16.hip", kernel_library("rocblas_f16"), {}, "-lrocblas")
+
+
+def build_rocblas_FP16_gemm_kernel():
+    print("Start building rocBLAS FP16 GEMM comparator ...")
+    failed = compile_many([rocblas_job()])
+    for out, err in failed:
+        print(f"Build failed: {out}\n{err}")
+    print("Build finished.")
+    return failed
 
 
 def build_Helix_MI355X_FP16_gemm_kernel():

@@ -6,7 +6,7 @@ import os
 
 from utils.helix_runtime import load
 from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
-from MI355X_FP32.build_MI355X_FP32 import library_for_key
+from MI355X_FP32.build_MI355X_FP32 import library_for_key, kernel_library
 from MI355X_FP32.profile_MI355X_FP32 import PROFILE_K, GEMV_PROFILE_K
 
 root_path = os.getcwd()
@@ -58,6 +58,15 @@ def get_MI355X_FP32_gemm_Helix_result(prof_dict, M, N, K, backend="hip"):
     tflops = 2 * M * N * K / 1e9 / cost
 
     return cost, tflops
+
+
+def get_MI355X_FP32_gemm_rocblas_result(M, N, K):
+    """The vendor library (rocblas_sgemm) on the same problem and operand layouts, timed the same way.
+    Mirrors get_Ampere_FP32_gemm_cublas_result (Ampere_FP32_gemm.py)."""
+    lib = load(kernel_library("rocblas_f32"))
+    _, avg, _ = lib.bench(M, N, K, warmup=10, iters=10, outer=1, rotate_bytes=0)
+    cost = avg * 1e3
+    return cost, 2 * M * N * K / 1e9 / cost
 
 
 def get_MI355X_FP32_gemm_Oracle_result(prof_dict, M, N, K):

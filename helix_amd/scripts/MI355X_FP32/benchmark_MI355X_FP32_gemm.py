@@ -5,7 +5,7 @@ import os
 
 from utils.get_benchmark_shape_list import get_gemm_op_MNKList
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP32.MI355X_FP32_gemm import get_MI355X_FP32_gemm_Helix_result
+from MI355X_FP32.MI355X_FP32_gemm import get_MI355X_FP32_gemm_Helix_result, get_MI355X_FP32_gemm_rocblas_result
 
 root_path = os.getcwd()
 
@@ -19,6 +19,15 @@ def MI355X_FP32_Helix_op_level_GEMM_benchmark(backend="hip"):
         print(f'{M}x{N}x{K}: Helix: {helix_tflops:.2f} TFLOPS')
 
 
+def MI355X_FP32_rocblas_op_level_GEMM_benchmark():
+    """Vendor column: mirrors Ampere_FP32_cublas_op_level_GEMM_benchmark (benchmark_Ampere_FP32_gemm.py)."""
+    MNKList = get_gemm_op_MNKList()
+    for M, N, K in MNKList:
+        _, rocblas_tflops = get_MI355X_FP32_gemm_rocblas_result(M, N, K)
+        print(f'{M}x{N}x{K}: rocblas: {rocblas_tflops:.2f} TFLOPS')
+
+
 if __name__ == "__main__":
 
     MI355X_FP32_Helix_op_level_GEMM_benchmark(backend="hip")
+    MI355X_FP32_rocblas_op_level_GEMM_benchmark()

@@ -5,7 +5,7 @@ import os
 
 from utils.get_benchmark_shape_list import get_llm_opset_MNKList, get_baseline_bert_MNKList
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP32.MI355X_FP32_gemm import get_MI355X_FP32_gemm_Helix_result
+from MI355X_FP32.MI355X_FP32_gemm import get_MI355X_FP32_gemm_Helix_result, get_MI355X_FP32_gemm_rocblas_result
 
 root_path = os.getcwd()
 
@@ -30,6 +30,19 @@ def MI355X_FP32_Helix_model_level_LLM_benchmark(backend="hip"):
     helix_GPT2_cost = _summed_cost(prof_dict, GPT2_MNKList, backend)
 
     print(f'Bert: {helix_Bert_cost:.2f} ms, LLAMA2: {helix_LLAMA2_cost:.2f} ms, GPT2: {helix_GPT2_cost:.2f} ms')
+
+
+def MI355X_FP32_rocblas_model_level_LLM_benchmark():
+    """Vendor column: mirrors Ampere_FP32_cublas_model_level_LLM_benchmark."""
+    costs = []
+    for MNKList in get_llm_opset_MNKList():
+        memo, total = {}, 0
+        for M, N, K in MNKList:
+            if (M, N, K) not in memo:
+                memo[(M, N, K)], _ = get_MI355X_FP32_gemm_rocblas_result(M, N, K)
+            total += memo[(M, N, K)]
+        costs.append(total)
+    print(f'Bert: {costs[0]:.2f} ms, LLAMA2: {costs[1]:.2f} ms, GPT2: {costs[2]:.2f} ms')
 
 
 def MI355X_FP32_Helix_baseline_bert_benchmark(backend="hip"):

@@ -39,20 +39,23 @@ def prof_dict_path(backend):
     return f"{root_path}/build/prof_dict/{backend}_cost_model.dict"
 
 
-def compile_command(src, out, defines):
+def compile_command(src, out, defines, link=""):
+    """hipcc line of one library; `link` holds extra linker flags (the vendor comparators' -lrocblas)."""
     inc = _find_include_dir()
     cmd = f"{HIPCC} {src} {COMPILE_OPTIONS} -I{inc} -I{os.path.join(SRC_ROOT, 'common')}"
     for k, v in defines.items():
         cmd += f" -D{k}={v}"
+    if link:
+        cmd += f" {link}"
     cmd += f" -o {out}"
     return cmd
 
 
-def compile_library(src, out, defines):
+def compile_library(src, out, defines, link=""):
     """Returns (ok, stderr_text)."""
     os.makedirs(os.path.dirname(out), exist_ok=True)
     tmp = out + ".tmp"
-    proc = subprocess.run(compile_command(src, tmp, defines), shell=True, capture_output=True, text=True)
+    proc = subprocess.run(compile_command(src, tmp, defines, link), shell=True, capture_output=True, text=True)
     if proc.returncode != 0:
         if os.path.exists(tmp):
             os.remove(tmp)
@@ -62,7 +65,7 @@ def compile_library(src, out, defines):
 
 
 def compile_many(jobs, max_workers=None, progress=None):
-    """jobs: iterable of (src, out, defines).  Compiles in parallel; returns list of failed outs."""
+    """jobs: iterable of (src, out, defines[, link flags]).  Compiles in parallel; returns list of failed outs."""
     jobs = list(jobs)
     if max_workers is None:
         max_workers = int(os.environ.get("MAX_JOBS", min(16, os.cpu_count() or 1)))

@@ -344,6 +344,25 @@ def test_conv_f16_baseline_layers_sampled():
 
 
 # ---------------------------------------------------------------------------------------------
+# vendor comparator libraries (rocBLAS behind the same C ABI)
+# ---------------------------------------------------------------------------------------------
+def test_rocblas_comparators_vs_oracle():
+    """The comparator libraries map the templates' operand layouts onto rocBLAS's column-major calls; a wrong
+    transpose or leading dimension fails here, before any benchmark prints a vendor column."""
+    lib16 = load(b16.kernel_library("rocblas_f16"))
+    for (M, N, K) in [(64, 48, 40), (300, 200, 136), (1, 7, 8), (130, 260, 1024)]:
+        A, B = seeded_inputs.gemm_operands(M, N, K, np.float16)
+        assert normwise(run_gemm_f16(lib16, A, B), O.hgemm_f32acc(A, B)) < TOL16, (M, N, K)
+    assert lib16.info()["family"] == "rocblas_f16"
+    lib32 = load(b32.kernel_library("rocblas_f32"))
+    for (M, N, K) in [(64, 48, 40), (152, 132, 97), (4, 8, 3), (260, 128, 1024)]:
+        A, B = seeded_inputs.gemm_operands(M, N, K, np.float32)
+        assert normwise(run_sgemm_f32(lib32, A, B), O.sgemm_seqk(A, B)) < TOL32, (M, N, K)
+    mn, avg, mx = lib16.bench(512, 512, 512, warmup=2, iters=3)
+    assert 0 < mn <= avg <= mx
+
+
+# ---------------------------------------------------------------------------------------------
 # FP32
 # ---------------------------------------------------------------------------------------------
 FP32_CONFIGS = [(128, 128, 16, 64, 64), (256, 128, 16, 128, 64), (32, 32, 8, 32, 32), (64, 256, 32, 32, 128),

@@ -211,8 +211,8 @@ def test_dispatch_tables_resolve():
 def test_cli_unsupported_combination_message():
     env = dict(os.environ, PYTHONPATH=os.path.join(ROOT, "helix_amd", "scripts"))
     out = subprocess.run([sys.executable, os.path.join(ROOT, "helix_amd", "scripts", "benchmark_op_level_eval.py"), "-o",
-                          "GEMM", "-b", "MI355X_FP16", "-s", "rocblas"], capture_output=True, text=True, env=env, cwd=ROOT)
-    assert out.returncode == 0 and out.stdout.strip() == "GEMM MI355X_FP16 rocblas is not supported"
+                          "Conv", "-b", "MI355X_FP16", "-s", "rocblas"], capture_output=True, text=True, env=env, cwd=ROOT)
+    assert out.returncode == 0 and out.stdout.strip() == "Conv MI355X_FP16 rocblas is not supported"
 
 
 # ---- C ABI ------------------------------------------------------------------------------------------------------
@@ -236,17 +236,17 @@ def test_every_built_library_exports_the_whole_abi():
         pytest.skip("kernel libraries are not built (run __graft_entry__.build())")
     want = set(_declared_symbols())
     # dlopen + dlsym only; no compute without a GPU.  A sample keeps this fast: every family, every 7th gemm
-    sample = [p for p in libs if "gemv" in p] + libs[::7]
+    sample = [p for p in libs if "gemv" in p or "rocblas" in p] + libs[::7]
     for path in sample:
         assert set(hip_ctypes.exported_symbols(path)) == want, path
         info = hip_ctypes.HelixLib(path).info()
-        assert info["arch"] == "gfx950" and info["family"] in ("gemm_f16", "gemv_f16", "sgemm_f32", "gemv_f32")
+        assert info["arch"] == "gfx950" and info["family"] in ("gemm_f16", "gemv_f16", "sgemm_f32", "gemv_f32", "rocblas_f16", "rocblas_f32")
 
 
 def test_all_expected_libraries_are_built():
     if not _built_libraries():
         pytest.skip("kernel libraries are not built (run __graft_entry__.build())")
-    missing = [out for (_, out, _) in b16.build_jobs() + b32.build_jobs() if not os.path.exists(out)]
+    missing = [job[1] for job in b16.build_jobs() + b32.build_jobs() if not os.path.exists(job[1])]
     assert not missing, missing[:5]
 
 
