@@ -29,16 +29,17 @@
 //     atomics, gemv_splitK.cu:213-217).
 //
 // MFMA variant (M >= MFMA_MIN_M)
-//   * a workgroup stages 16 activation rows of its K range (at most 2048 columns) in LDS, rows 16 bytes apart
-//     from a multiple of 256 so that 16 rows of one column sit in 16 different bank groups;
+//   * a workgroup walks its K range in chunks of MFMA_KCHUNK columns and stages 16 activation rows of the
+//     chunk in LDS, rows 16 bytes apart from a multiple of 256 so that 16 rows of one column sit in 16
+//     different bank groups;
 //   * a wave owns runs of 16 consecutive weight rows; per 256-wide K step it issues eight 16-byte loads per
 //     lane, straight into registers in the operand layout of the MFMA (lane l: row l % 16, columns 8*(l/16)
 //     .. +7 of a 32-wide block): 512 contiguous bytes per row and step, 64 per row and instruction; the same
 //     columns of activation row l % 16 come from LDS;
 //   * eight MFMAs per step accumulate the 16 x 16 block y[m][n]; steps are double-buffered; buffer bounds
 //     checking zero-fills weight rows beyond N;
-//   * K is partitioned over blockIdx.z into ranges of at most 2048 columns, and further until the launch has
-//     enough waves to cover the latency of the stream (FP32 workspace + fixed-order reduce).
+//   * K is partitioned over blockIdx.z only when the weight rows alone give the launch too few waves to cover
+//     the latency of the stream (FP32 workspace + fixed-order reduce).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -81,13 +82,13 @@
 #define MFMA_MIN_M 9        // activation rows from which the MFMA variant takes over (measured crossover)
 #endif
 #ifndef MFMA_TARGET_WAVES
-#define MFMA_TARGET_WAVES 4096
+#define MFMA_TARGET_WAVES 8192
 #endif
 #ifndef MFMA_WAVES_PER_BLOCK
-#define MFMA_WAVES_PER_BLOCK 8
+#define MFMA_WAVES_PER_BLOCK 4
 #endif
 #ifndef MFMA_KCHUNK
-#define MFMA_KCHUNK 1024    // widest K range of a workgroup of the MFMA variant (16 x MFMA_KCHUNK halves of LDS)
+#define MFMA_KCHUNK 1024    // columns of the 16 activation rows staged in LDS at a time by the MFMA variant
 #endif
 
 namespace {
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(64 * WPB) void helix_gemv_f16_kernel(const Params p
 // ---- MFMA variant -----------------------------------------------------------------------------------------
 constexpr int MSTEP = 256;                      // K extent of one step: eight 16-byte loads per lane, 512 bytes per weight row
 constexpr int MCH = MSTEP / 32;                 // 16-byte chunks per lane and step = MFMAs per step
-constexpr int MFMA_KCHUNK_MAX = MFMA_KCHUNK;     // K range of a workgroup: 16 staged activation rows of this width
+constexpr int MFMA_KCHUNK_MAX = MFMA_KCHUNK;     // staged columns: a multiple of MSTEP
 constexpr int MWPB = MFMA_WAVES_PER_BLOCK;
 constexpr int XROW_PAD = 16;                    // bytes between staged rows: 16 rows of one column hit 16 bank groups
 
@@ -335,6 +336,8 @@ __device__ __forceinline__ half8 buf_load8(__amdgpu_buffer_rsrc_t r, int voff, i
     return __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, MFMA_LOAD_AUX));
 }
 
+constexpr int MGROUPS = 4;                      // most 16-row groups one wave owns
+
 __global__ __launch_bounds__(64 * MWPB) void helix_gemv_f16_mfma_kernel(const Params p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
@@ -342,10 +345,10 @@ __global__ __launch_bounds__(64 * MWPB) void helix_gemv_f16_mfma_kernel(const Pa
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, q = lane >> 4;
     const int m0 = blockIdx.y * 16;
-    const int kchunk = p.kchunk;                                    // multiple of MSTEP
-    const int k_begin = (int)blockIdx.z * kchunk;
-    const int k_end = (k_begin + kchunk) < p.K ? (k_begin + kchunk) : p.K;
-    const int xrow = kchunk * 2 + XROW_PAD;                          // bytes per staged activation row
+    const int k_begin = (int)blockIdx.z * p.kchunk;                 // K range of this workgroup: a multiple of MSTEP
+    const int k_end = (k_begin + p.kchunk) < p.K ? (k_begin + p.kchunk) : p.K;
+    constexpr int XC = MFMA_KCHUNK_MAX;                              // columns staged at a time
+    constexpr int xrow = XC * 2 + XROW_PAD;                          // bytes per staged activation row
 
     const int ngroups = (p.N + 15) / 16;
     const int group_first = (blockIdx.x * MWPB + wave) * p.rows_per_wave;      // in units of 16-row groups
@@ -361,96 +364,94 @@ __global__ __launch_bounds__(64 * MWPB) void helix_gemv_f16_mfma_kernel(const Pa
                                                  (int)(((size_t)(rows_w - 1) * p.ldb + p.K) * 2), 0x00020000);
     };
     const int woff = (r * p.ldb + 8 * q) * 2;
-    auto load_step = [&](half8 (&w)[MCH], __amdgpu_buffer_rsrc_t rw, int k) {
-#pragma unroll
-        for (int c = 0; c < MCH; c++) w[c] = buf_load8(rw, woff + c * 64, k * 2);
-    };
-    auto load_step_tail = [&](half8 (&w)[MCH], __amdgpu_buffer_rsrc_t rw, int k) {
-#pragma unroll
-        for (int c = 0; c < MCH; c++) w[c] = buf_load8(rw, (k + 32 * c + 8 * q < k_end) ? woff + c * 64 : 0x7fffffff, k * 2);
-    };
-
-    // the first step of the first group is requested before the activations are staged
-    half8 wa[MCH], wb[MCH];
-    __amdgpu_buffer_rsrc_t rw = w_rsrc(group_first < ngroups ? group_first : 0);
-    const bool full_first = (k_begin + MSTEP <= k_end);
-    if (group_first < group_last) {
-        if (full_first) load_step(wa, rw, k_begin); else load_step_tail(wa, rw, k_begin);
-    }
-
-    // ---- stage the activations: 16 rows x kchunk, zero beyond M and beyond the K range --------------------
-    {
-        const int chunks_per_row = kchunk / 8;
-        const int total = 16 * chunks_per_row;
-        for (int c = tid; c < total; c += 64 * MWPB) {
-            const int m = c / chunks_per_row, kc = (c % chunks_per_row) * 8;
-            intx4 v = {0, 0, 0, 0};
-            if (m0 + m < p.M && k_begin + kc < k_end) v = *(const intx4*)(p.A + (size_t)(m0 + m) * p.lda + k_begin + kc);
-            *(intx4*)(smem + m * xrow + kc * 2) = v;
-        }
-    }
-    __syncthreads();
     const unsigned char* xl = smem + r * xrow + 8 * q * 2;           // this lane's activation row and column base
 
-    for (int g = group_first; g < group_last; g++) {
-        floatx4 acc = {0.f, 0.f, 0.f, 0.f};
-        auto mfma_step = [&](const half8 (&w)[MCH], int k) {
+    floatx4 acc[MGROUPS];
 #pragma unroll
-            for (int c = 0; c < MCH; c++) {
-                const half8 xv = *(const half8*)(xl + (k - k_begin) * 2 + c * 64);
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[c], xv, acc, 0, 0, 0);
-            }
-        };
-        // double-buffered steps: step s+1 is requested before the MFMAs of step s; wa holds the step at k
-        int k = k_begin;
-        for (; k + 3 * MSTEP <= k_end; k += 2 * MSTEP) {
-            load_step(wb, rw, k + MSTEP);
-            mfma_step(wa, k);
-            load_step(wa, rw, k + 2 * MSTEP);
-            mfma_step(wb, k + MSTEP);
-        }
-        // at most two steps and a partial one are left; wa holds the step at k
-        bool have_b = false;
-        if (k + MSTEP < k_end) {
-            if (k + 2 * MSTEP <= k_end) load_step(wb, rw, k + MSTEP); else load_step_tail(wb, rw, k + MSTEP);
-            have_b = true;
-        }
-        mfma_step(wa, k);
-        k += MSTEP;
-        if (have_b) {
-            if (k + MSTEP < k_end) {          // a third, partial step behind wb
-                load_step_tail(wa, rw, k + MSTEP);
-                mfma_step(wb, k);
-                mfma_step(wa, k + MSTEP);
-            } else {
-                mfma_step(wb, k);
-            }
-        }
-        // request the next group's first step, then store this group underneath it
-        if (g + 1 < group_last) {
-            rw = w_rsrc(g + 1);
-            if (full_first) load_step(wa, rw, k_begin); else load_step_tail(wa, rw, k_begin);
-        }
+    for (int gi = 0; gi < MGROUPS; gi++) acc[gi] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-        // lane l holds y[m0 + l % 16][n0 + 4*(l/16) + {0..3}]
+    // The K range is walked in chunks of XC columns: the workgroup stages 16 activation rows of the chunk in
+    // LDS, then every wave streams the chunk's columns of each of its row groups.
+    for (int kc = k_begin; kc < k_end; kc += XC) {
+        const int ce = (kc + XC) < k_end ? (kc + XC) : k_end;
+        __syncthreads();                                              // the previous chunk has been read
+        {
+            constexpr int chunks_per_row = XC / 8;
+            constexpr int total = 16 * chunks_per_row;
+            for (int c = tid; c < total; c += 64 * MWPB) {
+                const int m = c / chunks_per_row, kk = (c % chunks_per_row) * 8;
+                intx4 v = {0, 0, 0, 0};
+                if (m0 + m < p.M && kc + kk < ce) v = *(const intx4*)(p.A + (size_t)(m0 + m) * p.lda + kc + kk);
+                *(intx4*)(smem + m * xrow + kk * 2) = v;
+            }
+        }
+        __syncthreads();
+
+#pragma unroll
+        for (int gi = 0; gi < MGROUPS; gi++) {
+            const int g = group_first + gi;
+            if (g >= group_last) break;
+            const __amdgpu_buffer_rsrc_t rw = w_rsrc(g);
+            half8 wa[MCH], wb[MCH];
+            auto load_step = [&](half8 (&w)[MCH], int k) {
+                if (k + MSTEP <= ce) {
+#pragma unroll
+                    for (int c = 0; c < MCH; c++) w[c] = buf_load8(rw, woff + c * 64, k * 2);
+                } else {   // partial step: columns beyond the chunk read zeros
+#pragma unroll
+                    for (int c = 0; c < MCH; c++)
+                        w[c] = buf_load8(rw, (k + 32 * c + 8 * q < ce) ? woff + c * 64 : 0x7fffffff, k * 2);
+                }
+            };
+            auto mfma_step = [&](const half8 (&w)[MCH], int k) {
+#pragma unroll
+                for (int c = 0; c < MCH; c++) {
+                    const half8 xv = *(const half8*)(xl + (k - kc) * 2 + c * 64);
+                    acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[c], xv, acc[gi], 0, 0, 0);
+                }
+            };
+            // double-buffered steps: step s+1 is requested before the MFMAs of step s
+            load_step(wa, kc);
+            int k = kc;
+            for (; k + 2 * MSTEP < ce; k += 2 * MSTEP) {
+                load_step(wb, k + MSTEP);
+                mfma_step(wa, k);
+                load_step(wa, k + 2 * MSTEP);
+                mfma_step(wb, k + MSTEP);
+            }
+            if (k + MSTEP < ce) {
+                load_step(wb, k + MSTEP);
+                mfma_step(wa, k);
+                mfma_step(wb, k + MSTEP);
+            } else {
+                mfma_step(wa, k);
+            }
+        }
+    }
+
+    // lane l holds y[m0 + l % 16][n0 + 4*(l/16) + {0..3}] of each of its groups
+#pragma unroll
+    for (int gi = 0; gi < MGROUPS; gi++) {
+        const int g = group_first + gi;
+        if (g >= group_last) break;
         const int m = m0 + r, n = g * 16 + 4 * q;
         if (m < p.M && n < p.N) {
             if (p.ksplit > 1) {
                 float* dst = p.ws + ((size_t)blockIdx.z * p.M + m) * p.N + n;
-                if ((p.N & 3) == 0) *(floatx4*)dst = acc;
+                if ((p.N & 3) == 0) *(floatx4*)dst = acc[gi];
                 else
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        if (n + e < p.N) dst[e] = acc[e];
+                        if (n + e < p.N) dst[e] = acc[gi][e];
             } else {
                 half_t* dst = p.C + (size_t)m * p.ldc + n;
                 if ((p.ldc & 3) == 0 && (((uintptr_t)p.C) & 7) == 0 && n + 4 <= p.N) {
-                    half4 h = {(half_t)acc[0], (half_t)acc[1], (half_t)acc[2], (half_t)acc[3]};
+                    half4 h = {(half_t)acc[gi][0], (half_t)acc[gi][1], (half_t)acc[gi][2], (half_t)acc[gi][3]};
                     *(half4*)dst = h;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        if (n + e < p.N) dst[e] = (half_t)acc[e];
+                        if (n + e < p.N) dst[e] = (half_t)acc[gi][e];
                 }
             }
         }
@@ -495,18 +496,17 @@ inline const char* info_json() {
 constexpr int mtile_of(int M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
 // K partitioning: enough ranges that M_TILE activation rows of one range fit X_LDS_BYTES, at least SPLIT_K
-// MFMA variant: K ranges are multiples of 256 and at most 2048 wide (the staged activations), at least 512
-// wide, as many as bring the launch to about MFMA_TARGET_WAVES waves of 16 weight rows each, at least SPLIT_K
+// MFMA variant: K is partitioned only to give the launch enough waves (one wave owns up to MGROUPS groups of
+// 16 weight rows): ranges are multiples of 256, at least 1024 wide, at least SPLIT_K of them
 inline void k_partition_mfma(int N, int K, int* kchunk, int* ksplit) {
     const int steps = (K + MSTEP - 1) / MSTEP;
     const long long groups = (N + 15) / 16;
-    long long split = (MFMA_TARGET_WAVES + groups - 1) / groups;
-    const long long max_split = steps / 2 > 1 ? steps / 2 : 1;
+    long long split = (MFMA_TARGET_WAVES / 2 + groups - 1) / groups;     // aim for half the target before splitting
+    const long long max_split = steps / 4 > 1 ? steps / 4 : 1;
     if (split > max_split) split = max_split;
-    const long long min_split = (steps + MFMA_KCHUNK_MAX / MSTEP - 1) / (MFMA_KCHUNK_MAX / MSTEP);
-    if (split < min_split) split = min_split;
     if (split < SPLITK) split = SPLITK;
     if (split > steps) split = steps;
+    if (split < 1) split = 1;
     const int per = (int)((steps + split - 1) / split);
     *kchunk = per * MSTEP;
     *ksplit = (steps + per - 1) / per;
@@ -556,16 +556,14 @@ inline int launch_cfg(Params p, hipStream_t s) {
 inline int launch_mfma(Params p, hipStream_t s) {
     if ((long long)16 * p.ldb * 2 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
     const long long groups = (p.N + 15) / 16;
-    // 16-row groups per wave: as many as keep the launch near MFMA_TARGET_WAVES waves (the staged activations
-    // are shared by all groups a workgroup walks)
+    // 16-row groups per wave: as many (up to MGROUPS) as keep the launch near MFMA_TARGET_WAVES waves; the
+    // staged activations are shared by all groups a workgroup walks
     long long gpw = (groups * p.ksplit + MFMA_TARGET_WAVES - 1) / MFMA_TARGET_WAVES;
     if (gpw < 1) gpw = 1;
+    if (gpw > MGROUPS) gpw = MGROUPS;
     p.rows_per_wave = (int)gpw;
     const long long waves = (groups + gpw - 1) / gpw;
-    const int lds = 16 * (p.kchunk * 2 + XROW_PAD);
-    static int attr_rc = (int)hipFuncSetAttribute((const void*)helix_gemv_f16_mfma_kernel,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (attr_rc) return attr_rc;
+    const int lds = 16 * (MFMA_KCHUNK_MAX * 2 + XROW_PAD);
     dim3 grid((unsigned)((waves + MWPB - 1) / MWPB), (p.M + 15) / 16, p.ksplit), block(64 * MWPB);
     hipLaunchKernelGGL(helix_gemv_f16_mfma_kernel, grid, block, lds, s, p);
     return (int)hipGetLastError();
