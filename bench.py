@@ -44,19 +44,36 @@ def autotune(prof_keys, M, N, K):
 
 def gemv_rates(rotate_bytes=1 << 30):
     """Config 3: decode GEMV, cold (weights rotated through >= 1 GiB so the 256 MB last-level cache
-    cannot hold them).  Returns a list of dicts with achieved GB/s on the algorithmic bytes."""
+    cannot hold them).  Returns a list of dicts with achieved GB/s on the algorithmic bytes: the GEMV
+    library, and the fastest of the 32-row MFMA tile libraries on the same problem (the other family the cost
+    model chooses from for skinny shapes)."""
     from utils.helix_runtime import load
     from utils.roofline import gemm_bytes, HBM_BYTES_PER_S
     from utils.get_benchmark_shape_list import BASELINE_GEMV_BATCHES, BASELINE_GEMV_KN
-    from MI355X_FP16.build_MI355X_FP16 import kernel_library
+    from MI355X_FP16.build_MI355X_FP16 import kernel_library, library_for_key
+    from MI355X_FP16.profile_MI355X_FP16 import all_keys
     lib = load(kernel_library("gemv"))
+    tile_keys = [k for k in all_keys() if k[0] != 0 and k[1] == 32]
     out = []
     for (K, N) in BASELINE_GEMV_KN:
         for M in BASELINE_GEMV_BATCHES:
             mn, avg, _ = lib.bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)
             nbytes = gemm_bytes(M, N, K, 2)
-            out.append({"M": M, "K": K, "N": N, "us": round(mn * 1e6, 2), "GB/s": round(nbytes / mn / 1e9, 1),
-                        "frac_hbm_peak": round(nbytes / mn / HBM_BYTES_PER_S, 4)})
+            row = {"M": M, "K": K, "N": N, "us": round(mn * 1e6, 2), "GB/s": round(nbytes / mn / 1e9, 1),
+                   "frac_hbm_peak": round(nbytes / mn / HBM_BYTES_PER_S, 4)}
+            best_t, best_k = float("inf"), None
+            for k in tile_keys:
+                try:
+                    t = load(library_for_key(k)).bench(M, N, K, warmup=2, iters=10, outer=1, rotate_bytes=rotate_bytes)[1]
+                except Exception:
+                    continue
+                if t < best_t:
+                    best_t, best_k = t, k
+            if best_k is not None:
+                mn_t = load(library_for_key(best_k)).bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)[0]
+                row["tile_GB/s"] = round(nbytes / mn_t / 1e9, 1)
+                row["tile_config"] = list(best_k)
+            out.append(row)
     return out
 
 

@@ -9,7 +9,7 @@ here they are printed).  As there, split-K rows are left out of the two cost mod
 import os
 
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP16.MI355X_FP16_gemm import config_cost, run_config
+from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, run_config
 
 root_path = os.getcwd()
 
@@ -21,7 +21,7 @@ def cost_model(prof_dict, M, N, K, with_gemv=True):
     for k, v in prof_dict.items():
         if k[5] == 1 or (k[0] == 0 and not with_gemv):
             continue
-        cost = config_cost(k, v, M, N, K)
+        cost = config_cost(k, v, M, N, K, short_value(prof_dict, k))
         if min_cost > cost:
             min_cost, best_config = cost, k
     return best_config
@@ -41,7 +41,7 @@ def get_Helix_result(prof_dict, M, N, K):
 
 def get_gemv_result(prof_dict, M, N, K):
     gemv_keys = [k for k in prof_dict if k[0] == 0 and k[5] == 0]
-    k = min(gemv_keys, key=lambda k: config_cost(k, prof_dict[k], M, N, K))
+    k = min(gemv_keys, key=lambda k: config_cost(k, prof_dict[k], M, N, K, short_value(prof_dict, k)))
     return _tflops(k, M, N, K)
 
 

@@ -12,19 +12,31 @@ import os
 
 from utils.helix_runtime import load
 from MI355X_FP16.build_MI355X_FP16 import library_for_key
-from MI355X_FP16.MI355X_FP16_gemm import config_cost
+from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost
 
 root_path = os.getcwd()
 
 
+# Every column of output tiles gathers the im2col rows of its row block again (index arithmetic per
+# 16-byte chunk, which the plain GEMM the profile times does not have): measured over ResNet / GoogleNet /
+# AlexNet layers, a configuration's conv time exceeds its GEMM prediction by about this fraction per tile
+# column.
+GATHER_COST_PER_TILE_COLUMN = 0.2
+
+
+def conv_config_cost(k, v, M, N, K, v_short=None):
+    return config_cost(k, v, M, N, K, v_short) * (1.0 + GATHER_COST_PER_TILE_COLUMN * math.ceil(N / k[2]))
+
+
 def cost_model(prof_dict, M, N, K):
-    """GEMM cost model restricted to the MFMA configurations (the GEMV kernels have no conv path)."""
+    """GEMM cost model restricted to the MFMA configurations (the GEMV kernels have no conv path), with the
+    gather term above."""
     min_cost = float("inf")
     best_config = (1, 1, 1, 1, 1, 0, 32)
     for k, v in prof_dict.items():
         if k[0] == 0:
             continue
-        cost = config_cost(k, v, M, N, K)
+        cost = conv_config_cost(k, v, M, N, K, short_value(prof_dict, k))
         if min_cost > cost:
             min_cost = cost
             best_config = k

@@ -10,13 +10,17 @@ import os
 from utils.helix_runtime import load
 from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
 from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, SPLITK_MAX
-from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K
+from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K, PROFILE_K_SHORT
 
 root_path = os.getcwd()
 
-HBM_SUSTAINED_FRACTION = 0.6  # share of the datasheet HBM rate a streaming kernel sustains
-GEMV_LAUNCH_FLOOR_S = 3e-6
-SPLITK_REDUCE_LAUNCH_S = 4e-6  # the reduction kernel's launch, beyond what the profiled value already holds   # a kernel launch on an idle queue; keeps tiny problems from looking free
+HBM_SUSTAINED_FRACTION = 0.8  # share of the datasheet HBM rate a streaming kernel sustains
+GEMV_LAUNCH_FLOOR_S = 3.4e-6       # a kernel launch on an idle queue; keeps tiny problems from looking free
+GEMV_MFMA_FLOOR_S = 6.5e-6         # 9 or more activation rows: the K-partitioned MFMA variant plus its reduction
+GEMV_MFMA_MIN_M = 9                # MFMA_MIN_M of src_template/MI355X_FP16/gemv.hip
+GEMV_SPLITK_EXTRA_S = 2e-6         # the K-partitioned GEMV library's reduction pass on a problem too small to need it
+SPLITK_REDUCE_LAUNCH_S = 4e-6      # the reduction kernel's launch, beyond what the profiled value already holds
+ROUND_OVERLAP_S = 1e-6             # part of a round's fixed time that later rounds of one launch do not pay again
 
 
 def split_factor(k, M, N, K):
@@ -31,40 +35,61 @@ def split_factor(k, M, N, K):
     return max(s, 2)
 
 
-def config_cost(k, v, M, N, K):
-    """Predicted seconds of configuration k (profiled round time v) on an M x N x K problem.
+def round_time(v, v_short, K):
+    """Seconds of one round of tiles walking K: the line through the two profiled points (K_short, v_short)
+    and (K_profile, v); proportional to K, as the first version of this model was, when only the long point
+    exists."""
+    if v_short is None or not (v_short < float("inf")) or not (v < float("inf")):
+        return v * K / PROFILE_K
+    t = v_short + (v - v_short) * (K - PROFILE_K_SHORT) / (PROFILE_K - PROFILE_K_SHORT)
+    return max(t, 0.25 * v_short)
+
+
+def config_cost(k, v, M, N, K, v_short=None):
+    """Predicted seconds of configuration k (profiled round time v, and v_short at the short K when the
+    profile holds it) on an M x N x K problem.
 
     Reference form (Ampere_FP16_gemm.py:424-426): rounds = ceil(blocks / SMs), cost = rounds * v with
-    108 SMs and K ignored.  Here SMs -> 256 compute units and the round time is scaled by K / K_profile
-    (a round's time is proportional to the K extent each tile walks; split-K halves it)."""
+    108 SMs and K ignored.  Here SMs -> 256 compute units and the round time follows the K each tile walks
+    (split-K divides it)."""
     if k[0] == 0:
         # weight-streaming kernel: HBM-bound, so a partial round costs its share of a round (no
         # quantisation), never less than a launch; the streamed operand is the larger of M and N
         small, big = (M, N) if M <= N else (N, M)
         num_block = math.ceil(small / k[1]) * math.ceil(big / k[2])
-        return max(num_block / NUM_CU * v * max(K, 512) / PROFILE_K, GEMV_LAUNCH_FLOOR_S)
+        floor = GEMV_LAUNCH_FLOOR_S if small < GEMV_MFMA_MIN_M else GEMV_MFMA_FLOOR_S
+        cost = max(num_block / NUM_CU * v * max(K, 512) / PROFILE_K, floor)
+        return cost + (GEMV_SPLITK_EXTRA_S if k[5] == 1 else 0.0)
     splits = split_factor(k, M, N, K)
     num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * splits
     w = math.ceil(num_block / NUM_CU)
     # a tile walks K in whole BLOCK_K steps
-    k_scale = math.ceil(K / k[6]) * k[6] / PROFILE_K
+    k_walk = math.ceil(K / k[6]) * k[6]
     if k[5] == 1:
-        # the profiled value is two rounds of half-K partitions, i.e. about one full-K round; a round of
-        # this problem walks K / splits
-        k_scale = k_scale / splits + 64 / PROFILE_K
-    cost = w * v * k_scale
-    if k[5] == 1:
+        # the profiled value is two rounds of half-K partitions; a round of this problem walks K / splits
+        per_round = round_time(v, v_short, 2 * k_walk / splits) / 2
         # the FP32 partials are written and read back by a second kernel
-        cost += SPLITK_REDUCE_LAUNCH_S + (splits + 1) * M * N * 4 / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S)
+        extra = SPLITK_REDUCE_LAUNCH_S + (splits + 1) * M * N * 4 / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S)
+    else:
+        per_round = round_time(v, v_short, k_walk)
+        extra = 0.0
+    cost = w * per_round + extra
+    if v_short is not None:
+        cost -= ROUND_OVERLAP_S * (w - 1)
     # a tile round cannot beat streaming every operand once from HBM at the sustained rate
     return max(cost, gemm_bytes(M, N, K, 2) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
+
+
+def short_value(prof_dict, k):
+    """The short-K profile point of configuration k, or None (plain dicts, files without the second point)."""
+    return getattr(prof_dict, "short", {}).get(k)
 
 
 def cost_model(prof_dict, M, N, K):
     min_cost = float("inf")
     best_config = (1, 1, 1, 1, 1, 0, 32)
     for k, v in prof_dict.items():
-        cost = config_cost(k, v, M, N, K)
+        cost = config_cost(k, v, M, N, K, short_value(prof_dict, k))
         if min_cost > cost:
             min_cost = cost
             best_config = k

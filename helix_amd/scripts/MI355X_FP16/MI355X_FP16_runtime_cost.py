@@ -7,7 +7,7 @@ import time
 import os
 
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP16.MI355X_FP16_gemm import config_cost, run_config
+from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, run_config
 
 root_path = os.getcwd()
 
@@ -15,7 +15,7 @@ root_path = os.getcwd()
 def cost_model(prof_dict, M, N, K):
     cost_map = {}
     for k, v in prof_dict.items():
-        cost_map[k] = config_cost(k, v, M, N, K)
+        cost_map[k] = config_cost(k, v, M, N, K, short_value(prof_dict, k))
     best_config = min(cost_map, key=cost_map.get)
     return best_config
 

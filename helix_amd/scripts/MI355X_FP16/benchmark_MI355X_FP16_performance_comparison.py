@@ -6,7 +6,7 @@ import os
 
 from utils.get_benchmark_shape_list import get_gemm_op_MNKList
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP16.MI355X_FP16_gemm import config_cost, cost_model, run_config, get_MI355X_FP16_gemm_Oracle_result
+from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, cost_model, run_config, get_MI355X_FP16_gemm_Oracle_result
 
 root_path = os.getcwd()
 
@@ -17,7 +17,7 @@ def cost_model_static1(prof_dict, M, N, K):
     for k, v in prof_dict.items():
         if k[1] != k[3] or k[2] != k[4]:
             continue
-        cost = config_cost(k, v, M, N, K)
+        cost = config_cost(k, v, M, N, K, short_value(prof_dict, k))
         if min_cost > cost:
             min_cost = cost
             best_config = k

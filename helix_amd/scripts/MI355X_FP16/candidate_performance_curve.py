@@ -8,7 +8,7 @@ each line carries the candidate's own id.
 import os
 
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP16.MI355X_FP16_gemm import config_cost, run_config
+from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, run_config
 
 root_path = os.getcwd()
 
@@ -19,7 +19,7 @@ def get_all_candidate_performance(prof_dict, M, N, K):
     """Returns (best_id, best_config, [(id, config, tflops or None)]) and prints them."""
     min_cost, min_config, min_id = float("inf"), None, 0
     for id, (k, v) in enumerate(prof_dict.items(), start=1):
-        cost = config_cost(k, v, M, N, K)
+        cost = config_cost(k, v, M, N, K, short_value(prof_dict, k))
         if min_cost > cost:
             min_cost, min_config, min_id = cost, k, id
     print(f'Best candidate id: {min_id}, config = {min_config}')

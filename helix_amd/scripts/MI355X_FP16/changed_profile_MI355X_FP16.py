@@ -7,10 +7,10 @@ tile is multiplied by BLOCK_ROWS_SCALE * BLOCK_COLS_SCALE (:41).
 import os
 from tqdm import tqdm
 
-from utils.helix_runtime import write_prof_dict
+from utils.helix_runtime import write_prof_dict, ProfDict
 from MI355X_FP16.build_MI355X_FP16 import (K_STAGES_LIST, WAVE_TILE_LIST, BLOCK_SCALE_LIST, BLOCK_K_LIST,
                                            is_valid_config, SPLITK_STAGES_LIST)
-from MI355X_FP16.profile_MI355X_FP16 import time_config, GEMV_KEYS, GEMV_SPLITK_KEYS
+from MI355X_FP16.profile_MI355X_FP16 import time_config, GEMV_KEYS, GEMV_SPLITK_KEYS, PROFILE_K_SHORT
 
 root_path = os.getcwd()
 
@@ -19,7 +19,7 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
     if not os.path.exists(f"{root_path}/build/prof_dict"):
         os.makedirs(f"{root_path}/build/prof_dict")
 
-    prof_dict = {}
+    prof_dict = ProfDict()
     print("Start profiling MI355X FP16 GEMM kernel ...")
     total = len(K_STAGES_LIST) * len(WAVE_TILE_LIST) ** 2 * len(BLOCK_K_LIST) * 2 + 2
     with tqdm(total=total, desc="profiling") as pbar:
@@ -33,7 +33,9 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
                                 continue
                             if not is_valid_config(1, 1, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES):
                                 continue
-                            cost = time_config((K_STAGES, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K))
+                            base_key = (K_STAGES, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K)
+                            cost = time_config(base_key)
+                            cost_short = time_config(base_key, K=PROFILE_K_SHORT)
                             for BLOCK_ROWS_SCALE in BLOCK_SCALE_LIST:
                                 for BLOCK_COLS_SCALE in BLOCK_SCALE_LIST:
                                     BLOCK_ROWS = BLOCK_ROWS_SCALE * WAVE_ROWS
@@ -41,8 +43,9 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
                                     if not is_valid_config(BLOCK_ROWS_SCALE, BLOCK_COLS_SCALE, BLOCK_ROWS, BLOCK_COLS,
                                                            WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES):
                                         continue
-                                    prof_dict[(K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, splitK,
-                                               BLOCK_K)] = float(cost) * BLOCK_ROWS_SCALE * BLOCK_COLS_SCALE
+                                    key = (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K)
+                                    prof_dict[key] = float(cost) * BLOCK_ROWS_SCALE * BLOCK_COLS_SCALE
+                                    prof_dict.short[key] = float(cost_short) * BLOCK_ROWS_SCALE * BLOCK_COLS_SCALE
 
         for key in GEMV_KEYS + GEMV_SPLITK_KEYS:
             prof_dict[key] = time_config(key)

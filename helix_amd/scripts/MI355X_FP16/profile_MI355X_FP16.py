@@ -6,18 +6,20 @@ Mirrors scripts/Ampere_FP16/profile_Ampere_FP16.py:17-62.  The reference times o
 nor L2 contention, so here every configuration is timed on one full round of tiles over the 256 compute
 units (16 x 16 tiles): the cost model's `ceil(blocks / 256) * value` then has the reference's meaning
 (rounds x time per round), and a one-round problem is predicted with its launch and pipeline-fill
-latency included.
+latency included.  Every MFMA configuration is timed a second time at a short K (PROFILE_K_SHORT), stored in
+a second dict file: the two points give the cost model a round's fixed part and its per-K part.
 """
 import os
 from tqdm import tqdm
 
-from utils.helix_runtime import load, write_prof_dict
+from utils.helix_runtime import load, write_prof_dict, ProfDict
 from utils.roofline import NUM_CU
 from MI355X_FP16.build_MI355X_FP16 import iter_configs, library_for_key, SPLITK_STAGES_LIST
 
 root_path = os.getcwd()
 
 PROFILE_K = 4096            # reference: K = 4096 for every GEMM tile (profile_Ampere_FP16.py:36)
+PROFILE_K_SHORT = 512       # second point: launch + pipeline fill + epilogue dominate at this K
 PROFILE_ROUNDS = 1          # rounds of 256 tiles in the timed problem
 PROFILE_GRID = 16           # 16 x 16 = 256 tiles = one tile per compute unit
 # GEMV rows keep the reference's tag (first field 0, profile_Ampere_FP16.py:51,57) and its
@@ -31,16 +33,16 @@ GEMV_KEY, GEMV_SPLITK_KEY = GEMV_KEYS[0], GEMV_SPLITK_KEYS[0]
 GEMV_PROFILE_ROWS = 128 * NUM_CU   # one 128-row block per compute unit
 
 
-def profile_problem(key):
+def profile_problem(key, K=PROFILE_K):
     """(M, N, K) of the timed problem and the number of 256-tile rounds it holds."""
     if key[0] == 0:
-        return key[1], GEMV_PROFILE_ROWS, PROFILE_K, 1
-    return key[1] * PROFILE_GRID, key[2] * PROFILE_GRID * PROFILE_ROUNDS, PROFILE_K, PROFILE_ROUNDS
+        return key[1], GEMV_PROFILE_ROWS, K, 1
+    return key[1] * PROFILE_GRID, key[2] * PROFILE_GRID * PROFILE_ROUNDS, K, PROFILE_ROUNDS
 
 
-def time_config(key, warmup=3, iters=10):
-    """Seconds for one round of 256 tiles of this configuration (inf if it cannot run)."""
-    M, N, K, rounds = profile_problem(key)
+def time_config(key, warmup=3, iters=10, K=PROFILE_K):
+    """Seconds for one round of 256 tiles of this configuration at this K (inf if it cannot run)."""
+    M, N, K, rounds = profile_problem(key, K)
     try:
         lib = load(library_for_key(key))
         rotate = (1 << 30) if key[0] == 0 else 0
@@ -66,12 +68,14 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
     if not os.path.exists(f"{root_path}/build/prof_dict"):
         os.makedirs(f"{root_path}/build/prof_dict")
 
-    prof_dict = {}
+    prof_dict = ProfDict()
     print("Start profiling MI355X FP16 GEMM kernel ...")
     keys = all_keys()
     with tqdm(total=len(keys), desc="profiling") as pbar:
         for key in keys:
             prof_dict[key] = time_config(key)
+            if key[0] != 0:
+                prof_dict.short[key] = time_config(key, K=PROFILE_K_SHORT)
             pbar.update(1)
 
     write_prof_dict("MI355X_FP16", prof_dict)

@@ -7,7 +7,7 @@ import os
 
 from utils.helix_runtime import load
 from MI355X_FP32.build_MI355X_FP32 import library_for_key
-from MI355X_FP32.MI355X_FP32_gemm import config_cost
+from MI355X_FP32.MI355X_FP32_gemm import config_cost, extra_points
 
 root_path = os.getcwd()
 
@@ -18,7 +18,7 @@ def cost_model(prof_dict, M, N, K):
     for k, v in prof_dict.items():
         if k[2] == 0:
             continue
-        cost = config_cost(k, v, M, N, K)
+        cost = config_cost(k, v, M, N, K, extra_points(prof_dict, k))
         if min_cost > cost:
             min_cost = cost
             best_config = k

@@ -7,31 +7,66 @@ import os
 from utils.helix_runtime import load
 from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
 from MI355X_FP32.build_MI355X_FP32 import library_for_key, kernel_library
-from MI355X_FP32.profile_MI355X_FP32 import PROFILE_K, GEMV_PROFILE_K
+from MI355X_FP32.profile_MI355X_FP32 import PROFILE_K, PROFILE_K_SHORT, GEMV_PROFILE_K
 
 root_path = os.getcwd()
 
-HBM_SUSTAINED_FRACTION = 0.6
-GEMV_LAUNCH_FLOOR_S = 3e-6
+HBM_SUSTAINED_FRACTION = 0.8
+GEMV_LAUNCH_FLOOR_S = 3.4e-6
+GEMV_SPLITK_EXTRA_S = 2e-6        # the K-partitioned library's reduction pass on a problem too small to need it
+# a further round of tiles costs what the two-round profile shows beyond one round, but never less than this
+# share of a lone round: the profiled problems sit in the caches, long ones do not
+LATER_ROUND_MIN_SHARE = 0.5
+# rate at which the compute units take A and B tiles in (bytes of M*N*K*4*(1/BM + 1/BN) per second): what the
+# small-tile configurations reach on 2048^3 ... 8192^3
+OPERAND_BYTES_PER_S = 6.5e12
 
 
-def config_cost(k, v, M, N, K):
+def _line(x0, y0, x1, y1, x):
+    return y0 + (y1 - y0) * (x - x0) / (x1 - x0)
+
+
+def _finite(*values):
+    return all(v is not None and v < float("inf") for v in values)
+
+
+def config_cost(k, v, M, N, K, points=None):
     """rounds * time-per-round as in Ampere_FP32_gemm.py:93-95, with 256 compute units for 108 SMs and
-    the round time scaled by K / K_profile (the reference ignores K)."""
+    the round time following K (the reference ignores K).  `points` = (short, two_rounds, short_two_rounds)
+    of the profile when it holds them: then the first round costs the line through the two one-round points
+    and each further round the line through the two-round increments."""
     if k[2] == 0:
         small, big = (M, N) if M <= N else (N, M)
         num_block = math.ceil(small / k[0]) * math.ceil(big / k[1])
-        return max(num_block / NUM_CU * v * max(K, 256) / GEMV_PROFILE_K, GEMV_LAUNCH_FLOOR_S)
-    num_block = math.ceil(M / k[0]) * math.ceil(N / k[1])
-    w = math.ceil(num_block / NUM_CU)
-    return max(w * v * max(K, 32) / PROFILE_K, gemm_bytes(M, N, K, 4) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
+        cost = max(num_block / NUM_CU * v * max(K, 256) / GEMV_PROFILE_K, GEMV_LAUNCH_FLOOR_S)
+        return cost + (GEMV_SPLITK_EXTRA_S if k[5] == 1 else 0.0)
+    tiles_m, tiles_n = math.ceil(M / k[0]), math.ceil(N / k[1])
+    w = math.ceil(tiles_m * tiles_n / NUM_CU)
+    hbm_floor = gemm_bytes(M, N, K, 4) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S)
+    if points is None or not _finite(v, *points):
+        return max(w * v * max(K, 32) / PROFILE_K, hbm_floor)
+    short, two, short_two = points
+    k_walk = math.ceil(K / k[2]) * k[2]
+    first = max(_line(PROFILE_K_SHORT, short, PROFILE_K, v, k_walk), 0.25 * short)
+    later = _line(PROFILE_K_SHORT, short_two - short, PROFILE_K, two - v, k_walk)
+    later = min(max(later, LATER_ROUND_MIN_SHARE * first), first)
+    operand_floor = 4.0 * tiles_m * k[0] * tiles_n * k[1] * K * (1 / k[0] + 1 / k[1]) / OPERAND_BYTES_PER_S
+    return max(first + (w - 1) * later, hbm_floor, operand_floor)
+
+
+def extra_points(prof_dict, k):
+    """(short, two_rounds, short_two_rounds) of configuration k, or None when the profile lacks any of them."""
+    try:
+        return (prof_dict.short[k], prof_dict.two_rounds[k], prof_dict.short_two_rounds[k])
+    except (AttributeError, KeyError):
+        return None
 
 
 def cost_model(prof_dict, M, N, K):
     min_cost = float("inf")
     best_config = (1, 1, 1, 1, 1, 1, 1, 1)
     for k, v in prof_dict.items():
-        cost = config_cost(k, v, M, N, K)
+        cost = config_cost(k, v, M, N, K, extra_points(prof_dict, k))
         if min_cost > cost:
             min_cost = cost
             best_config = k

@@ -96,18 +96,57 @@ def load(path):
     return lib
 
 
-def read_prof_dict(backend):
-    with open(prof_dict_path(backend), "r") as f:
+# extra profile points kept beside the reference's dict: attribute of ProfDict -> file name suffix
+EXTRA_PROFILE_POINTS = {"short": "shortK", "two_rounds": "2rounds", "short_two_rounds": "shortK_2rounds"}
+
+
+class ProfDict(dict):
+    """{config tuple: seconds per round of tiles at the profile K}, the reference's dict, plus optional
+    extra points for the same keys, each {} when its file is absent:
+      .short             one round at a short K: separates a round's fixed part (launch, pipeline fill,
+                         epilogue) from its per-K part;
+      .two_rounds        two rounds at the profile K (whole launch, not per round);
+      .short_two_rounds  two rounds at the short K: what a further round costs once workgroups of
+                         consecutive rounds share a compute unit."""
+
+    def __init__(self, *a, **kw):
+        super().__init__(*a, **kw)
+        for attr in EXTRA_PROFILE_POINTS:
+            setattr(self, attr, {})
+
+
+def extra_prof_dict_path(backend, suffix):
+    return f"{root_path}/build/prof_dict/{backend}_cost_model_{suffix}.dict"
+
+
+def _read_dict_file(path):
+    with open(path, "r") as f:
         lines = f.readlines()
         # same `eval(lines[0])` as the reference (benchmark_Ampere_FP16_gemm.py:10-12); `inf` is bound because
         # skipped configurations are stored as float('inf'), whose repr is not a Python literal
         return eval(lines[0], {"inf": float("inf"), "nan": float("nan")})
 
 
+def read_prof_dict(backend):
+    prof_dict = ProfDict(_read_dict_file(prof_dict_path(backend)))
+    for attr, suffix in EXTRA_PROFILE_POINTS.items():
+        if os.path.exists(extra_prof_dict_path(backend, suffix)):
+            setattr(prof_dict, attr, _read_dict_file(extra_prof_dict_path(backend, suffix)))
+    return prof_dict
+
+
 def write_prof_dict(backend, prof_dict):
     os.makedirs(os.path.dirname(prof_dict_path(backend)), exist_ok=True)
     with open(prof_dict_path(backend), "w") as f:
-        f.write(str(prof_dict))
+        f.write(str(dict(prof_dict)))
+    for attr, suffix in EXTRA_PROFILE_POINTS.items():
+        path = extra_prof_dict_path(backend, suffix)
+        extra = getattr(prof_dict, attr, None)
+        if extra:
+            with open(path, "w") as f:
+                f.write(str(dict(extra)))
+        elif os.path.exists(path):
+            os.remove(path)   # never pair a new profile with stale extra points
 
 
 def reference_line(M, N, K, min_s, avg_s, max_s):

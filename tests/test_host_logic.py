@@ -138,6 +138,62 @@ def test_fp32_cost_model_hand_cases():
     assert g32.config_cost((128, 128, 16, 64, 64, 2, 4, 4), 1.0, 4096, 4096, 2 * K) == pytest.approx(8.0)
 
 
+def test_fp16_cost_model_two_point_profile():
+    """With the short-K point a round costs the line through (K_short, v_short) and (K_profile, v); a further
+    round of one launch saves ROUND_OVERLAP_S of the fixed part."""
+    K, Ks = p16.PROFILE_K, p16.PROFILE_K_SHORT
+    small, big = (2, 32, 64, 32, 32, 0, 64), (2, 128, 256, 64, 64, 0, 64)
+    # per-K slopes favour the small tile (per tile area), fixed parts favour the big one
+    d = helix_runtime.ProfDict({small: 17e-6, big: 60e-6})
+    d.short = {small: 4e-6, big: 8e-6}
+    assert g16.round_time(17e-6, 4e-6, Ks) == pytest.approx(4e-6)
+    assert g16.round_time(17e-6, 4e-6, K) == pytest.approx(17e-6)
+    assert g16.round_time(17e-6, 4e-6, (K + Ks) // 2) == pytest.approx(10.5e-6)
+    assert g16.round_time(17e-6, None, K // 2) == pytest.approx(8.5e-6)                 # one point: proportional
+    assert g16.round_time(17e-6, 4e-6, 64) >= 1e-6                                       # never below a quarter of the short point
+    # 100352 x 256 x 64 (a 1x1 convolution as GEMM): 12544 small tiles = 49 rounds, 784 big tiles = 4 rounds
+    c_small = g16.config_cost(small, d[small], 100352, 256, 64, d.short[small])
+    c_big = g16.config_cost(big, d[big], 100352, 256, 64, d.short[big])
+    r_small, r_big = g16.round_time(17e-6, 4e-6, 64), g16.round_time(60e-6, 8e-6, 64)
+    assert c_small == pytest.approx(49 * r_small - 48 * g16.ROUND_OVERLAP_S)
+    assert c_big == pytest.approx(max(4 * r_big - 3 * g16.ROUND_OVERLAP_S,
+                                      roofline.gemm_bytes(100352, 256, 64, 2) / (g16.HBM_SUSTAINED_FRACTION * roofline.HBM_BYTES_PER_S)))
+    assert g16.cost_model(d, 100352, 256, 64) == big
+    # without the short point a round is taken to cost K / K_profile of the profiled one: 49 almost free rounds
+    assert g16.config_cost(small, d[small], 100352, 256, 64) == pytest.approx(49 * 17e-6 * 64 / K)
+    # conv: every column of tiles gathers its rows again
+    assert c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6) == \
+        pytest.approx(g16.config_cost(big, 60e-6, 4096, 512, K, 8e-6) * (1 + 2 * c16.GATHER_COST_PER_TILE_COLUMN))
+    # GEMV rows: 9 or more activation rows run the K-partitioned MFMA variant (higher floor); the split-K
+    # GEMV library pays its reduction
+    assert g16.config_cost((0, 16, 128, 0, 0, 0, 0), 1e-9, 13, 128, 512) == g16.GEMV_MFMA_FLOOR_S
+    assert g16.config_cost((0, 16, 128, 0, 0, 1, 0), 1e-9, 4, 128, 512) == \
+        pytest.approx(g16.GEMV_LAUNCH_FLOOR_S + g16.GEMV_SPLITK_EXTRA_S)
+
+
+def test_fp32_cost_model_extra_points():
+    K, Ks = p32.PROFILE_K, p32.PROFILE_K_SHORT
+    key = (64, 64, 16, 32, 32, 2, 4, 4)
+    d = helix_runtime.ProfDict({key: 30e-6})
+    d.short, d.two_rounds, d.short_two_rounds = {key: 12e-6}, {key: 48e-6}, {key: 15e-6}
+    pts = g32.extra_points(d, key)
+    assert pts == (12e-6, 48e-6, 15e-6)
+    assert g32.extra_points({key: 1.0}, key) is None
+    # one round of 256 tiles: the one-round line; 1024 x 1024 outputs with 64 x 64 tiles
+    assert g32.config_cost(key, 30e-6, 1024, 1024, K, pts) == pytest.approx(30e-6)
+    assert g32.config_cost(key, 30e-6, 1024, 1024, Ks, pts) == pytest.approx(12e-6)
+    # four rounds at the profile K: later rounds cost the two-round increment (18 us, above half of 30 us)
+    assert g32.config_cost(key, 30e-6, 2048, 2048, K, pts) == pytest.approx(30e-6 + 3 * 18e-6)
+    # at the short K the increment (3 us) is below half a lone round (6 us), so the share applies
+    assert g32.config_cost(key, 30e-6, 2048, 2048, Ks, pts) == pytest.approx(12e-6 + 3 * 6e-6)
+    # a long problem on small tiles is bound by the rate the compute units take operands in
+    big = g32.config_cost(key, 20e-6, 8192, 8192, 8192, (12e-6, 30e-6, 15e-6))
+    assert big == pytest.approx(4.0 * 8192 ** 3 * (2 / 64) / g32.OPERAND_BYTES_PER_S)
+    # the K-partitioned GEMV library pays its reduction
+    assert g32.config_cost((4, 128, 0, 0, 0, 1, 4, 4), 1e-9, 2, 128, 256) == \
+        pytest.approx(g32.GEMV_LAUNCH_FLOOR_S + g32.GEMV_SPLITK_EXTRA_S)
+
+
 def test_padded_k():
     assert g16.padded_k(770) == 776 and g16.padded_k(768) == 768 and g16.padded_k(1) == 8
 
@@ -160,6 +216,18 @@ def test_prof_dict_roundtrip(tmp_path, monkeypatch):
     # (eval(lines[0]), benchmark_Ampere_FP16_gemm.py:10-12), with inf defined
     assert "inf" in text
     assert helix_runtime.read_prof_dict("MI355X_FP16") == d
+    assert helix_runtime.read_prof_dict("MI355X_FP16").short == {}
+    # extra profile points travel in files of their own beside the reference's dict
+    pd = helix_runtime.ProfDict(d)
+    pd.short = {(2, 128, 128, 64, 64, 0, 64): 4e-6}
+    pd.two_rounds = {(2, 128, 128, 64, 64, 0, 64): 2.5e-5}
+    helix_runtime.write_prof_dict("MI355X_FP16", pd)
+    assert open(tmp_path / "build" / "prof_dict" / "MI355X_FP16_cost_model.dict").read() == text
+    back = helix_runtime.read_prof_dict("MI355X_FP16")
+    assert back == d and back.short == pd.short and back.two_rounds == pd.two_rounds and back.short_two_rounds == {}
+    # a profile without them removes the stale files
+    helix_runtime.write_prof_dict("MI355X_FP16", d)
+    assert helix_runtime.read_prof_dict("MI355X_FP16").short == {}
 
 
 def test_shape_lists():
