@@ -42,38 +42,21 @@ def autotune(prof_keys, M, N, K):
     return best, best_t, tried
 
 
-def gemv_rates(rotate_bytes=1 << 30):
-    """Config 3: decode GEMV, cold (weights rotated through >= 1 GiB so the 256 MB last-level cache
-    cannot hold them).  Returns a list of dicts with achieved GB/s on the algorithmic bytes: the GEMV
-    library, and the fastest of the 32-row MFMA tile libraries on the same problem (the other family the cost
-    model chooses from for skinny shapes)."""
-    from utils.helix_runtime import load
-    from utils.roofline import gemm_bytes, HBM_BYTES_PER_S
-    from utils.get_benchmark_shape_list import BASELINE_GEMV_BATCHES, BASELINE_GEMV_KN
-    from MI355X_FP16.build_MI355X_FP16 import kernel_library, library_for_key
-    from MI355X_FP16.profile_MI355X_FP16 import all_keys
-    lib = load(kernel_library("gemv"))
-    tile_keys = [k for k in all_keys() if k[0] != 0 and k[1] == 32]
-    out = []
-    for (K, N) in BASELINE_GEMV_KN:
-        for M in BASELINE_GEMV_BATCHES:
-            mn, avg, _ = lib.bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)
-            nbytes = gemm_bytes(M, N, K, 2)
-            row = {"M": M, "K": K, "N": N, "us": round(mn * 1e6, 2), "GB/s": round(nbytes / mn / 1e9, 1),
-                   "frac_hbm_peak": round(nbytes / mn / HBM_BYTES_PER_S, 4)}
-            best_t, best_k = float("inf"), None
-            for k in tile_keys:
-                try:
-                    t = load(library_for_key(k)).bench(M, N, K, warmup=2, iters=10, outer=1, rotate_bytes=rotate_bytes)[1]
-                except Exception:
-                    continue
-                if t < best_t:
-                    best_t, best_k = t, k
-            if best_k is not None:
-                mn_t = load(library_for_key(best_k)).bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)[0]
-                row["tile_GB/s"] = round(nbytes / mn_t / 1e9, 1)
-                row["tile_config"] = list(best_k)
-            out.append(row)
+def other_configs():
+    """The other measured configurations, each against its roofline: decode GEMV (cold, HBM), FP32 squares, the
+    batch-32 ResNet-50 conv layers and the BERT-base GEMM list, through the cost model's picks (profiles first
+    when no dict is on disk).  Rows as printed by helix_amd/scripts/benchmark_baseline_configs.py."""
+    import benchmark_baseline_configs as bc
+    out = {}
+    be16 = bc.Backend("MI355X_FP16")
+    d16 = be16.prof_dict()
+    out["gemv_hbm"] = bc.gemv_rows(be16, d16)
+    out["conv_f16"] = bc.conv_rows(be16, d16)
+    out["bert_f16"] = bc.bert_rows(be16, d16)[-1]
+    be32 = bc.Backend("MI355X_FP32")
+    d32 = be32.prof_dict()
+    out["sgemm_f32"] = bc.square_rows(be32, d32)
+    out["bert_f32"] = bc.bert_rows(be32, d32)[-1]
     return out
 
 
@@ -102,7 +85,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-gemv", action="store_true")
+    ap.add_argument("--no-gemv", action="store_true",
+                    help="skip the other configurations (decode GEMV, FP32 squares, conv layers, BERT list)")
     ap.add_argument("--kernel-config", type=str, default=None,
                     help="skip the template search and time this configuration, e.g. 2,256,256,64,128,0,64")
     ap.add_argument("--operands", choices=["seeded", "zeros"], default="seeded",
@@ -218,7 +202,7 @@ def main():
         torch.cuda.synchronize()
         out["torch_matmul_tflops"] = round(flops / ((time.perf_counter() - t0) / args.steps) / 1e12, 2)
     if not args.no_gemv:
-        out["gemv_hbm"] = gemv_rates()
+        out.update(other_configs())
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

@@ -1,0 +1,157 @@
+"""python3 benchmark_baseline_configs.py -c {square,gemv,conv,bert,all} -b <backend> [--oracle] [--json]
+
+The measured configurations of this backend, each against the roofline that bounds it:
+  square  M = N = K in {1024, 2048, 4096, 8192}                              (MFMA peak)
+  gemv    decode shapes, M in {1, 4, 16} activation rows, weights cold       (HBM peak)
+  conv    batch-32 NHWC ResNet-50-shaped layers, implicit GEMM               (MFMA peak and HBM peak)
+  bert    BERT-base encoder GEMMs at 4096 tokens x 12 layers + 4000x2300x770 (MFMA peak)
+Every row is run through the cost model's pick (what the reference's benchmark wrappers do,
+scripts/Ampere_FP16/benchmark_Ampere_FP16_gemm.py:9-30); --oracle adds the exhaustive per-shape search
+(benchmark_Ampere_FP16_performance_comparison.py:56-69).  Needs build_template.py to have run; profiles
+first when no cost-model dict is on disk.
+"""
+import argparse
+import importlib
+import json
+import os
+
+from _dispatch import MI355X_BACKENDS
+from utils import roofline as R
+from utils import get_benchmark_shape_list as S
+from utils.helix_runtime import load, read_prof_dict, prof_dict_path
+
+
+class Backend:
+    """The per-backend functions this script needs, looked up by the reference's naming scheme."""
+
+    def __init__(self, name):
+        self.name = name
+        self.fp32 = name.endswith("FP32")
+        self.elem_bytes = 4 if self.fp32 else 2
+        self.peak = R.FP32_MFMA_FLOPS if self.fp32 else R.FP16_MFMA_FLOPS
+        mod = lambda m: importlib.import_module(f"{name}.{m}")
+        self.gemm, self.conv, self.build, self.profile = (mod(f"{name}_gemm"), mod(f"{name}_conv"),
+                                                         mod(f"build_{name}"), mod(f"profile_{name}"))
+        self.gemm_result = getattr(self.gemm, f"get_{name}_gemm_Helix_result")
+        self.gemm_oracle = getattr(self.gemm, f"get_{name}_gemm_Oracle_result")
+        self.conv_result = getattr(self.conv, f"get_{name}_conv_Helix_result")
+
+    def prof_dict(self):
+        if not os.path.exists(prof_dict_path(self.name)):
+            getattr(self.profile, f"profile_Helix_{self.name}_gemm_kernel")()
+        return read_prof_dict(self.name)
+
+    def is_gemv_key(self, k):
+        return (k[2] == 0) if self.fp32 else (k[0] == 0)
+
+    def block_rows(self, k):
+        return k[0] if self.fp32 else k[1]
+
+
+def square_rows(be, prof_dict, oracle=False):
+    rows = []
+    for s in S.BASELINE_SQUARE_SIZES:
+        key = be.gemm.cost_model(prof_dict, s, s, s)
+        ms, tflops = be.gemm_result(prof_dict, s, s, s)
+        row = {"M": s, "N": s, "K": s, "config": list(key), "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
+               "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
+        if oracle:
+            oms, otf, okey = be.gemm_oracle(prof_dict, s, s, s)
+            row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2),
+                        "oracle_frac_mfma_peak": round(otf * 1e12 / be.peak, 4)})
+        rows.append(row)
+    return rows
+
+
+def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
+    """Weights rotated through >= 1 GiB so the 256 MB last-level cache cannot hold them.  Per shape: the GEMV
+    library, and (tiles=True) the fastest of the 32-row MFMA tile libraries, the other family the cost model
+    chooses from for skinny shapes."""
+    lib = load(be.build.kernel_library("gemv_fp32" if be.fp32 else "gemv"))
+    tile_keys = [k for k in prof_dict if not be.is_gemv_key(k) and be.block_rows(k) == 32] if tiles else []
+    rows = []
+    for (K, N) in S.BASELINE_GEMV_KN:
+        for M in S.BASELINE_GEMV_BATCHES:
+            mn, _, _ = lib.bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)
+            nbytes = R.gemm_bytes(M, N, K, be.elem_bytes)
+            row = {"M": M, "K": K, "N": N, "us": round(mn * 1e6, 2), "GB/s": round(nbytes / mn / 1e9, 1),
+                   "frac_hbm_peak": round(nbytes / mn / R.HBM_BYTES_PER_S, 4)}
+            best_t, best_k = float("inf"), None
+            for k in tile_keys:
+                try:
+                    t = load(be.build.library_for_key(k)).bench(M, N, K, warmup=2, iters=10, outer=1,
+                                                               rotate_bytes=rotate_bytes)[1]
+                except Exception:
+                    continue
+                if t < best_t:
+                    best_t, best_k = t, k
+            if best_k is not None:
+                mn_t = load(be.build.library_for_key(best_k)).bench(M, N, K, warmup=5, iters=50, outer=3,
+                                                                   rotate_bytes=rotate_bytes)[0]
+                row["tile_GB/s"] = round(nbytes / mn_t / 1e9, 1)
+                row["tile_config"] = list(best_k)
+            rows.append(row)
+    return rows
+
+
+def conv_rows(be, prof_dict):
+    rows = []
+    for shp in S.get_baseline_conv_shape_list():
+        b, ic, h, w, oc, kh, kw, st, pd = shp
+        M = b * ((h + 2 * pd - kh) // st + 1) * ((w + 2 * pd - kw) // st + 1)
+        key = be.conv.cost_model(prof_dict, M, oc, ic * kh * kw)
+        ms, tflops = be.conv_result(prof_dict, *shp)
+        nbytes = R.conv_bytes(*shp, be.elem_bytes)
+        rows.append({"shape": list(shp), "gemm_MNK": [M, oc, ic * kh * kw], "config": list(key), "us": round(ms * 1e3, 2),
+                     "TFLOP/s": round(tflops, 2), "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4),
+                     "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
+                     "frac_hbm_peak": round(nbytes / (ms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
+    return rows
+
+
+def bert_rows(be, prof_dict):
+    """Per distinct GEMM of the encoder, then the whole list (12 layers + the irregular shape) as one row."""
+    memo, rows = {}, []
+    total_ms, total_flops = 0.0, 0.0
+    for (M, N, K) in S.get_baseline_bert_MNKList():
+        if (M, N, K) not in memo:
+            memo[(M, N, K)] = be.gemm_result(prof_dict, M, N, K)
+            ms, tflops = memo[(M, N, K)]
+            rows.append({"M": M, "N": N, "K": K, "config": list(be.gemm.cost_model(prof_dict, M, N, K)),
+                         "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
+                         "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)})
+        total_ms += memo[(M, N, K)][0]
+        total_flops += 2.0 * M * N * K
+    tf = total_flops / (total_ms * 1e-3) / 1e12
+    rows.append({"total_ms": round(total_ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf * 1e12 / be.peak, 4)})
+    return rows
+
+
+SECTIONS = {"square": square_rows, "gemv": gemv_rows, "conv": conv_rows, "bert": bert_rows}
+
+
+def run(backend, configs, oracle=False):
+    be = Backend(backend)
+    prof_dict = be.prof_dict()
+    out = {}
+    for name in configs:
+        out[name] = square_rows(be, prof_dict, oracle) if name == "square" else SECTIONS[name](be, prof_dict)
+    return out
+
+
+if __name__ == "__main__":
+    parser = argparse.ArgumentParser(description="Benchmark the measured configurations against their rooflines")
+    parser.add_argument("-c", "--config", type=str, choices=list(SECTIONS) + ["all"], default="all")
+    parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default="MI355X_FP16")
+    parser.add_argument("--oracle", action="store_true", help="also run the exhaustive search on the square shapes")
+    parser.add_argument("--json", action="store_true", help="one JSON object instead of the table")
+    args = parser.parse_args()
+
+    result = run(args.backend, list(SECTIONS) if args.config == "all" else [args.config], args.oracle)
+    if args.json:
+        print(json.dumps(result))
+    else:
+        for name, rows in result.items():
+            print(f"== {name} ({args.backend})")
+            for row in rows:
+                print("  " + ", ".join(f"{k}: {v}" for k, v in row.items()))

@@ -276,6 +276,24 @@ def test_dispatch_tables_resolve():
             assert callable(_dispatch.resolve(row))
 
 
+def test_baseline_config_script_resolves_backend_functions():
+    import benchmark_baseline_configs as bc
+    for name, fp32 in (("MI355X_FP16", False), ("MI355X_FP32", True)):
+        be = bc.Backend(name)
+        assert be.fp32 == fp32 and be.elem_bytes == (4 if fp32 else 2)
+        assert be.peak == (roofline.FP32_MFMA_FLOPS if fp32 else roofline.FP16_MFMA_FLOPS)
+        assert callable(be.gemm_result) and callable(be.gemm_oracle) and callable(be.conv_result)
+    be16, be32 = bc.Backend("MI355X_FP16"), bc.Backend("MI355X_FP32")
+    assert be16.is_gemv_key((0, 4, 128, 0, 0, 0, 0)) and not be16.is_gemv_key((2, 32, 64, 32, 32, 0, 128))
+    assert be32.is_gemv_key((4, 128, 0, 0, 0, 0, 4, 4)) and not be32.is_gemv_key((32, 64, 16, 32, 32, 2, 4, 4))
+    assert be16.block_rows((2, 32, 64, 32, 32, 0, 128)) == 32 and be32.block_rows((32, 64, 16, 32, 32, 2, 4, 4)) == 32
+    assert set(bc.SECTIONS) == {"square", "gemv", "conv", "bert"}
+    out = subprocess.run([sys.executable, os.path.join(ROOT, "helix_amd", "scripts", "benchmark_baseline_configs.py"),
+                          "-c", "nothing"], capture_output=True, text=True,
+                         env=dict(os.environ, PYTHONPATH=os.path.join(ROOT, "helix_amd", "scripts")))
+    assert out.returncode == 2 and "invalid choice" in out.stderr
+
+
 def test_cli_unsupported_combination_message():
     env = dict(os.environ, PYTHONPATH=os.path.join(ROOT, "helix_amd", "scripts"))
     out = subprocess.run([sys.executable, os.path.join(ROOT, "helix_amd", "scripts", "benchmark_op_level_eval.py"), "-o",
