@@ -1,4 +1,4 @@
-"""python3 benchmark_baseline_configs.py -c {square,gemv,conv,bert,all} -b <backend> [--oracle] [--json]
+"""python3 benchmark_baseline_configs.py -c {square,gemv,conv,bert,all} -b <backend> [--oracle] [--no-tiles] [--json]
 
 The measured configurations of this backend, each against the roofline that bounds it:
   square  M = N = K in {1024, 2048, 4096, 8192}                              (MFMA peak)
@@ -130,12 +130,17 @@ def bert_rows(be, prof_dict):
 SECTIONS = {"square": square_rows, "gemv": gemv_rows, "conv": conv_rows, "bert": bert_rows}
 
 
-def run(backend, configs, oracle=False):
+def run(backend, configs, oracle=False, tiles=True):
     be = Backend(backend)
     prof_dict = be.prof_dict()
     out = {}
     for name in configs:
-        out[name] = square_rows(be, prof_dict, oracle) if name == "square" else SECTIONS[name](be, prof_dict)
+        if name == "square":
+            out[name] = square_rows(be, prof_dict, oracle)
+        elif name == "gemv":
+            out[name] = gemv_rows(be, prof_dict, tiles=tiles)
+        else:
+            out[name] = SECTIONS[name](be, prof_dict)
     return out
 
 
@@ -144,10 +149,12 @@ if __name__ == "__main__":
     parser.add_argument("-c", "--config", type=str, choices=list(SECTIONS) + ["all"], default="all")
     parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default="MI355X_FP16")
     parser.add_argument("--oracle", action="store_true", help="also run the exhaustive search on the square shapes")
+    parser.add_argument("--no-tiles", action="store_true", help="gemv: time the GEMV library only")
     parser.add_argument("--json", action="store_true", help="one JSON object instead of the table")
     args = parser.parse_args()
 
-    result = run(args.backend, list(SECTIONS) if args.config == "all" else [args.config], args.oracle)
+    result = run(args.backend, list(SECTIONS) if args.config == "all" else [args.config], args.oracle,
+                 tiles=not args.no_tiles)
     if args.json:
         print(json.dumps(result))
     else:

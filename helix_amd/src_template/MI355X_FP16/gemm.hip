@@ -103,8 +103,32 @@ static_assert(STAGES == 2, "K_STAGES: one K tile staged in registers behind the 
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
 static_assert(SPLITK >= 1 && SPLITK <= 8, "SPLIT_K out of range");
 
+// Division by a run-time constant as multiply and shift: q = (n * mul) >> shift is floor(n / d) for every
+// 0 <= n < 2^31 when shift = 31 + ceil(log2 d) and mul = floor(2^shift / d) + 1 (the error term
+// n * (d - 2^shift mod d) / 2^shift stays below 1).  The gather decomposes output rows and K indices with
+// it instead of the forty-odd instructions of a general integer division.
+struct FastDiv {
+    unsigned mul;
+    int shift;
+    int d;
+    __host__ __device__ __forceinline__ int div(int n) const {
+        return (int)(((unsigned long long)(unsigned)n * mul) >> shift);
+    }
+};
+
+inline FastDiv make_fastdiv(int d) {
+    int l = 0;
+    while ((1LL << l) < d) l++;
+    FastDiv f;
+    f.shift = 31 + l;
+    f.mul = (unsigned)(((1ULL << f.shift) / (unsigned long long)d) + 1ULL);
+    f.d = d;
+    return f;
+}
+
 struct ConvGeom {
     int H, W, IC, OH, OW, kW, stride, pad, M;  // M = batch*OH*OW
+    FastDiv by_OW, by_OH, by_IC, by_kW;
 };
 
 struct Params {
@@ -284,34 +308,66 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
 #pragma unroll
         for (int i = 0; i < A_ITERS; i++) {
             const int m = m0 + r0 + i * ROWS_PER_ITER;
-            const int ow = m % p.g.OW;
-            const int t = m / p.g.OW;
-            const int oh = t % p.g.OH;
-            const int b = t / p.g.OH;
+            const int t = p.g.by_OW.div(m);
+            const int ow = m - t * p.g.OW;
+            const int b = p.g.by_OH.div(t);
+            const int oh = t - b * p.g.OH;
             cv_img[i] = (m < p.g.M) ? b * p.g.H * p.g.W : -1;
             cv_ih[i] = oh * p.g.stride - p.g.pad;
             cv_iw[i] = ow * p.g.stride - p.g.pad;
             if (MODE == 2) {
                 cv_base[i] = ((cv_img[i] + cv_ih[i] * p.g.W + cv_iw[i]) * p.g.IC + gch_a[i] * 8) * 2;
+                // taps inside the image form a rectangle kh in [kh_lo, kh_hi) x kw in [kw_lo, kw_hi)
+                const int kH = p.g.by_kW.div(p.g.by_IC.div(p.K));
+                const int kw_lo = cv_iw[i] < 0 ? -cv_iw[i] : 0;
+                const int kw_hi = (p.g.W - cv_iw[i]) < p.g.kW ? (p.g.W - cv_iw[i]) : p.g.kW;
+                const int kh_lo = cv_ih[i] < 0 ? -cv_ih[i] : 0;
+                const int kh_hi = (p.g.H - cv_ih[i]) < kH ? (p.g.H - cv_ih[i]) : kH;
+                const unsigned row_bits = (kw_hi > kw_lo && cv_img[i] >= 0) ? ((1u << kw_hi) - (1u << kw_lo)) : 0u;
                 unsigned taps = 0;
-                const int ntaps = p.K / p.g.IC;
-                for (int t = 0; t < ntaps; t++) {
-                    const int ih = cv_ih[i] + t / p.g.kW, iw = cv_iw[i] + t % p.g.kW;
-                    if (cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W) taps |= 1u << t;
-                }
+                for (int kh = 0; kh < kH; kh++)
+                    if (kh >= kh_lo && kh < kh_hi) taps |= row_bits << (kh * p.g.kW);
                 cv_taps[i] = taps;
             }
         }
     }
 
-    // MODE 2: scalar state of the K tile at k0: byte offset of its filter tap and channel block, and its tap bit
+    // MODE 2: scalar state of a K tile: byte offset of its filter tap and channel block, and its tap bit.
+    // K tiles are visited in order, so the state is stepped from tile to tile (a tile never straddles a tap:
+    // IC is a multiple of BLOCK_K) instead of being derived from k0 with integer divisions every tile.
     struct ConvTile { int soff; unsigned tapbit; };
-    auto conv_tile = [&](int k0) -> ConvTile {
+    struct ConvWalk {
+        int k0, c0, kw, tap, tap_off;   // tile start, channel within the tap, tap column, tap index, tap byte offset
+    };
+    ConvWalk walk{0, 0, 0, 0, 0};
+    if (MODE == 2) {
+        const int tap = p.g.by_IC.div(k_begin), kh = p.g.by_kW.div(tap);
+        walk.k0 = k_begin;
+        walk.c0 = k_begin - tap * p.g.IC;
+        walk.kw = tap - kh * p.g.kW;
+        walk.tap = tap;
+        walk.tap_off = (kh * p.g.W + walk.kw) * p.g.IC * 2;
+    }
+    // state of the tile the walk stands on (empty past the end of K), then one tile forward
+    auto conv_next = [&]() -> ConvTile {
         ConvTile ct{0, 0u};
-        if (MODE == 2 && k0 < p.K) {
-            const int tap = k0 / p.g.IC, c0 = k0 % p.g.IC;
-            ct.soff = (((tap / p.g.kW) * p.g.W + tap % p.g.kW) * p.g.IC + c0) * 2;
-            ct.tapbit = 1u << tap;
+        if (MODE == 2) {
+            if (walk.k0 < p.K) {
+                ct.soff = walk.tap_off + walk.c0 * 2;
+                ct.tapbit = 1u << walk.tap;
+            }
+            walk.k0 += BK;
+            walk.c0 += BK;
+            if (walk.c0 >= p.g.IC) {
+                walk.c0 = 0;
+                walk.tap += 1;
+                walk.kw += 1;
+                walk.tap_off += p.g.IC * 2;
+                if (walk.kw == p.g.kW) {
+                    walk.kw = 0;
+                    walk.tap_off += (p.g.W - p.g.kW) * p.g.IC * 2;
+                }
+            }
         }
         return ct;
     };
@@ -326,10 +382,10 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             return (cv_taps[i] & ct.tapbit) ? cv_base[i] + ct.soff : OOB_OFFSET;
         } else {
             const int k = k0 + gch_a[i] * 8;  // k = (kh*kW + kw)*IC + c, 8 consecutive c per chunk
-            const int c = k % p.g.IC;
-            const int t = k / p.g.IC;
-            const int kw = t % p.g.kW;
-            const int kh = t / p.g.kW;
+            const int t = p.g.by_IC.div(k);
+            const int c = k - t * p.g.IC;
+            const int kh = p.g.by_kW.div(t);
+            const int kw = t - kh * p.g.kW;
             const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
             const bool ok = !(narrow && gch_a[i] * 8 >= width) && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 &&
                             iw < p.g.W;
@@ -414,14 +470,14 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         // prologue: tile 0 into the staging registers and on to LDS, the registers refilled with tile 1
         {
             const __amdgpu_buffer_rsrc_t ra = rsrc_a(k_begin, true), rb = rsrc_b(k_begin, true);
-            const ConvTile ct = conv_tile(k_begin);
+            const ConvTile ct = conv_next();
 #pragma unroll
             for (int idx = 0; idx < NV; idx++) st[idx] = load_slot(idx, k_begin, true, first_w, ra, rb, ct);
         }
         {
             const int k0 = tile_k0(1);
             const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0, 1 < ktiles), rb = rsrc_b(k0, 1 < ktiles);
-            const ConvTile ct = conv_tile(k0);
+            const ConvTile ct = conv_next();
 #pragma unroll
             for (int idx = 0; idx < NV; idx++) {
                 store_slot(idx, 0, st[idx]);
@@ -444,15 +500,13 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     }
 
     // Slots [LO, HI) of K tile kt, multiplied from LDS stage `stage`.
-    auto tile_part = [&](auto lo_c, auto hi_c, int kt, int stage) {
+    // k0c, ra, rb, ctc: start, descriptors and conv state of tile kt + 2, the one loaded into the staging
+    // registers once they are written.
+    auto tile_part = [&](auto lo_c, auto hi_c, int stage, int k0c, __amdgpu_buffer_rsrc_t ra,
+                         __amdgpu_buffer_rsrc_t rb, ConvTile ctc) {
         constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
         const unsigned char* sb = smem + stage * STAGE_BYTES;
         const unsigned char* sb_nxt = smem + (stage ^ 1) * STAGE_BYTES;
-        const int kt_ld = kt + 2;                  // tile loaded into the staging registers once they are written
-        const int k0c = tile_k0(kt_ld);
-        // past the last tile the loads still issue, with empty descriptors, which keeps the body branch-free
-        const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0c, kt_ld < ktiles), rb = rsrc_b(k0c, kt_ld < ktiles);
-        const ConvTile ctc = conv_tile(k0c);
 #pragma unroll
         for (int n = LO / T_RES; n < (HI + T_RES - 1) / T_RES; n++) {   // streamed fragment n: k-step s, index u
 #pragma unroll
@@ -490,11 +544,16 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     constexpr std::integral_constant<int, G> c_end{};
     int stage = 0;
     for (int kt = 0; kt < ktiles; kt++) {
-        tile_part(c_0, c_bar, kt, stage);
+        const int kt_ld = kt + 2;
+        const int k0c = tile_k0(kt_ld);
+        // past the last tile the loads still issue, with empty descriptors, which keeps the body branch-free
+        const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0c, kt_ld < ktiles), rb = rsrc_b(k0c, kt_ld < ktiles);
+        const ConvTile ctc = conv_next();
+        tile_part(c_0, c_bar, stage, k0c, ra, rb, ctc);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        tile_part(c_bar, c_end, kt, stage);
+        tile_part(c_bar, c_end, stage, k0c, ra, rb, ctc);
         stage ^= 1;
     }
 
@@ -741,9 +800,10 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
     p.tiles_m = (int)((M + BM - 1) / BM); p.tiles_n = (OC + BN - 1) / BN;
     p.a_bytes = (unsigned)xbytes;
     p.splits = split_factor(M, OC, K);
-    p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M};
+    p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M,
+                   make_fastdiv(OW), make_fastdiv(OH), make_fastdiv(IC), make_fastdiv(kW)};
     // a K tile inside one filter tap (and a tap mask that fits 32 bits) takes the scalar-tap gather
-    if (IC % BK == 0 && kH * kW <= 32) return launch<2>(p, ws, ws_bytes, s);
+    if (IC % BK == 0 && kH * kW <= 32 && kW < 32) return launch<2>(p, ws, ws_bytes, s);
     return launch<1>(p, ws, ws_bytes, s);
 }
 
