@@ -42,6 +42,7 @@
 
 #include "helix_abi.h"
 #include "helix_im2col.h"
+#include "helix_fastdiv.h"
 
 #ifndef BLOCK_ROWS
 #define BLOCK_ROWS 256
@@ -103,28 +104,7 @@ static_assert(STAGES == 2, "K_STAGES: one K tile staged in registers behind the 
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
 static_assert(SPLITK >= 1 && SPLITK <= 8, "SPLIT_K out of range");
 
-// Division by a run-time constant as multiply and shift: q = (n * mul) >> shift is floor(n / d) for every
-// 0 <= n < 2^31 when shift = 31 + ceil(log2 d) and mul = floor(2^shift / d) + 1 (the error term
-// n * (d - 2^shift mod d) / 2^shift stays below 1).  The gather decomposes output rows and K indices with
-// it instead of the forty-odd instructions of a general integer division.
-struct FastDiv {
-    unsigned mul;
-    int shift;
-    int d;
-    __host__ __device__ __forceinline__ int div(int n) const {
-        return (int)(((unsigned long long)(unsigned)n * mul) >> shift);
-    }
-};
-
-inline FastDiv make_fastdiv(int d) {
-    int l = 0;
-    while ((1LL << l) < d) l++;
-    FastDiv f;
-    f.shift = 31 + l;
-    f.mul = (unsigned)(((1ULL << f.shift) / (unsigned long long)d) + 1ULL);
-    f.d = d;
-    return f;
-}
+using helix_fastdiv::FastDiv;   // division by a run-time constant as multiply and shift
 
 struct ConvGeom {
     int H, W, IC, OH, OW, kW, stride, pad, M;  // M = batch*OH*OW
@@ -801,7 +781,7 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
     p.a_bytes = (unsigned)xbytes;
     p.splits = split_factor(M, OC, K);
     p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M,
-                   make_fastdiv(OW), make_fastdiv(OH), make_fastdiv(IC), make_fastdiv(kW)};
+                   helix_fastdiv::make(OW), helix_fastdiv::make(OH), helix_fastdiv::make(IC), helix_fastdiv::make(kW)};
     // a K tile inside one filter tap (and a tap mask that fits 32 bits) takes the scalar-tap gather
     if (IC % BK == 0 && kH * kW <= 32 && kW < 32) return launch<2>(p, ws, ws_bytes, s);
     return launch<1>(p, ws, ws_bytes, s);

@@ -21,6 +21,7 @@
 
 #include "helix_abi.h"
 #include "helix_im2col.h"
+#include "helix_fastdiv.h"
 
 #ifndef BM
 #define BM 128
@@ -68,8 +69,11 @@ static_assert((BK * A_CPR) % NTHREADS == 0 && (BK * B_CPR) % NTHREADS == 0, "til
 static_assert((BM * K_CPR) % NTHREADS == 0 && (BN * K_CPR) % NTHREADS == 0, "conv tile copy must divide evenly");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
 
+using helix_fastdiv::FastDiv;   // division by a run-time constant as multiply and shift
+
 struct ConvGeom {
     int H, W, IC, OH, OW, kW, stride, pad, M;
+    FastDiv by_OW, by_OH, by_IC, by_kW;
 };
 
 struct Params {
@@ -128,10 +132,10 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 #pragma unroll
         for (int i = 0; i < NA; i++) {
             const int m = m0 + (tid + i * NTHREADS) / K_CPR;
-            const int ow = m % p.g.OW;
-            const int t = m / p.g.OW;
-            const int oh = t % p.g.OH;
-            const int b = t / p.g.OH;
+            const int t = p.g.by_OW.div(m);
+            const int ow = m - t * p.g.OW;
+            const int b = p.g.by_OH.div(t);
+            const int oh = t - b * p.g.OH;
             cv_img[i] = (m < p.g.M) ? b * p.g.H * p.g.W : -1;
             cv_ih[i] = oh * p.g.stride - p.g.pad;
             cv_iw[i] = ow * p.g.stride - p.g.pad;
@@ -160,10 +164,10 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
             const int kc = tid % K_CPR;
             const int k = k0 + kc * 4;
             const bool dead = k >= p.K;
-            const int c = k % p.g.IC;
-            const int t = k / p.g.IC;
-            const int kw = t % p.g.kW;
-            const int kh = t / p.g.kW;
+            const int t = p.g.by_IC.div(k);
+            const int c = k - t * p.g.IC;
+            const int kh = p.g.by_kW.div(t);
+            const int kw = t - kh * p.g.kW;
 #pragma unroll
             for (int i = 0; i < NA; i++) {
                 const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
@@ -376,7 +380,8 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
     p.M = (int)M; p.N = OC; p.K = (int)K; p.lda = 0; p.ldb = (int)K; p.ldc = OC;
     p.tiles_m = (int)((M + BM - 1) / BM); p.tiles_n = (OC + BN - 1) / BN;
     p.a_bytes = (unsigned)xbytes;
-    p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M};
+    p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M,
+                   helix_fastdiv::make(OW), helix_fastdiv::make(OH), helix_fastdiv::make(IC), helix_fastdiv::make(kW)};
     return launch<true>(p, s);
 }
 

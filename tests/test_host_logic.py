@@ -194,6 +194,19 @@ def test_fp32_cost_model_extra_points():
         pytest.approx(g32.GEMV_LAUNCH_FLOOR_S + g32.GEMV_SPLITK_EXTRA_S)
 
 
+def test_fastdiv_header_matches_integer_division(tmp_path):
+    """The conv gathers divide by OW, OH, IC and kW with a multiply and a shift (common/helix_fastdiv.h); the
+    host half of the header is compiled and swept against `/` here."""
+    exe = str(tmp_path / "fastdiv_check")
+    src = os.path.join(ROOT, "tests", "cpp", "fastdiv_check.cpp")
+    inc = os.path.join(ROOT, "helix_amd", "src_template", "common")
+    build = subprocess.run(["hipcc", "-O2", "-w", "--offload-arch=gfx950", f"-I{inc}", src, "-o", exe],
+                           capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr[-2000:]
+    run = subprocess.run([exe], capture_output=True, text=True)
+    assert run.returncode == 0 and "mismatches 0" in run.stdout, run.stdout + run.stderr
+
+
 def test_padded_k():
     assert g16.padded_k(770) == 776 and g16.padded_k(768) == 768 and g16.padded_k(1) == 8
 
