@@ -7,7 +7,7 @@ names modulo the backend tag.  Differences that follow from the target:
   * output is build/bin_fp16/lib<kernel>_<params>.so exporting the C ABI of include/helix_abi.h instead of
     an executable; the convolution path lives in the same library as the GEMM of each configuration
     (implicit GEMM), so there is no im2col artifact;
-  * wave tiles are multiples of 32x32 (2x2 of the 16x16x32 MFMA tile), K_STAGE becomes K_STAGES (the
+  * wave tiles are multiples of 32 rows x 16 columns of the 16x16x32 MFMA tile, K_STAGE becomes K_STAGES (the
     pipeline holds the K tile being multiplied in LDS and one more on its way through registers: 2 is the
     only depth the gfx950 template implements), and BLOCK_K is a template parameter too (it is fixed to 32
     in the reference, gemm.cu:77);
@@ -23,7 +23,11 @@ root_path = os.getcwd()
 K_STAGES_LIST = [2]
 SPLITK_MAX = 8              # a split-K library partitions K 2 .. 8 ways, chosen per problem
 SPLITK_STAGES_LIST = [2]    # pipeline depths a split-K variant is built for
-WAVE_TILE_LIST = [32, 64, 128]
+WAVE_TILE_LIST = [32, 64, 128]              # wave-tile rows (the epilogue pairs 16-row MFMA tiles)
+# wave-tile columns: 48 and 96 give block tiles of 96 and 192 columns, which divide the 768 / 2304 / 3072-wide
+# transformer projections into whole rounds of 256 tiles where the powers of two leave a quarter of the
+# compute units idle
+WAVE_COLS_LIST = [32, 48, 64, 96, 128]
 BLOCK_SCALE_LIST = [1, 2, 4]
 BLOCK_K_LIST = [64, 128]
 LDS_LIMIT = 160 * 1024
@@ -64,6 +68,11 @@ def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, 
         return False
     if threads % chunks_per_row:
         return False
+    # the streamed operand's fragments of a K tile go through a window of 2 * min(fragments, 2) registers
+    tm, tn = wave_rows // 16, wave_cols // 16
+    streamed = tn if tm > tn else tm
+    if ((block_k // 32) * streamed) % (2 * min(streamed, 2)):
+        return False
     waves_per_simd = (threads // 64 + 3) // 4
     if vgpr_estimate(block_rows, block_cols, wave_rows, wave_cols, block_k) > VGPR_FILE // waves_per_simd:
         return False
@@ -74,7 +83,7 @@ def iter_configs():
     """Yields (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in build order."""
     for K_STAGES in K_STAGES_LIST:
         for WAVE_ROWS in WAVE_TILE_LIST:
-            for WAVE_COLS in WAVE_TILE_LIST:
+            for WAVE_COLS in WAVE_COLS_LIST:
                 for BLOCK_ROWS_SCALE in BLOCK_SCALE_LIST:
                     for BLOCK_COLS_SCALE in BLOCK_SCALE_LIST:
                         for BLOCK_K in BLOCK_K_LIST:

@@ -8,7 +8,7 @@ import os
 from tqdm import tqdm
 
 from utils.helix_runtime import write_prof_dict, ProfDict
-from MI355X_FP16.build_MI355X_FP16 import (K_STAGES_LIST, WAVE_TILE_LIST, BLOCK_SCALE_LIST, BLOCK_K_LIST,
+from MI355X_FP16.build_MI355X_FP16 import (K_STAGES_LIST, WAVE_TILE_LIST, WAVE_COLS_LIST, BLOCK_SCALE_LIST, BLOCK_K_LIST,
                                            is_valid_config, SPLITK_STAGES_LIST)
 from MI355X_FP16.profile_MI355X_FP16 import time_config, GEMV_KEYS, GEMV_SPLITK_KEYS, PROFILE_K_SHORT
 
@@ -21,11 +21,11 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
 
     prof_dict = ProfDict()
     print("Start profiling MI355X FP16 GEMM kernel ...")
-    total = len(K_STAGES_LIST) * len(WAVE_TILE_LIST) ** 2 * len(BLOCK_K_LIST) * 2 + 2
+    total = len(K_STAGES_LIST) * len(WAVE_TILE_LIST) * len(WAVE_COLS_LIST) * len(BLOCK_K_LIST) * 2 + 2
     with tqdm(total=total, desc="profiling") as pbar:
         for K_STAGES in K_STAGES_LIST:
             for WAVE_ROWS in WAVE_TILE_LIST:
-                for WAVE_COLS in WAVE_TILE_LIST:
+                for WAVE_COLS in WAVE_COLS_LIST:
                     for BLOCK_K in BLOCK_K_LIST:
                         for splitK in (0, 1):
                             pbar.update(1)

@@ -96,7 +96,7 @@ constexpr int STRIP_BYTES = 32 * STRIP_LD;
 constexpr int LDS_BYTES = RING_BYTES > NWAVES * STRIP_BYTES ? RING_BYTES : NWAVES * STRIP_BYTES;
 
 static_assert(BM % WM == 0 && BN % WN == 0, "block tile must be a multiple of the wave tile");
-static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32 x 32");
+static_assert(WM % 32 == 0 && WN % 16 == 0, "wave tile: rows in multiples of 32 (the epilogue pairs 16-row tiles), columns of 16");
 static_assert(BK == 64 || BK == 128, "BLOCK_K holds an even number of 32-wide MFMA k-steps: 64 or 128");
 static_assert(NTHREADS <= 1024 && NTHREADS % KCH == 0, "bad thread count");
 static_assert((BM * KCH) % NTHREADS == 0 && (BN * KCH) % NTHREADS == 0, "tile copy must divide evenly");

@@ -77,7 +77,10 @@ def run_sgemm_f32(lib, A, B):
 
 FP16_CONFIGS = [(2, 256, 256, 128, 128, 64), (2, 256, 256, 64, 128, 64), (2, 128, 128, 64, 64, 128), (2, 64, 64, 32, 32, 64),
                 (2, 32, 32, 32, 32, 128), (2, 256, 64, 64, 32, 64), (2, 64, 256, 32, 128, 128), (2, 128, 256, 128, 64, 64),
-                (2, 128, 128, 64, 64, 64), (2, 256, 256, 128, 64, 64), (2, 64, 64, 32, 32, 128), (2, 32, 128, 32, 64, 64)]
+                (2, 128, 128, 64, 64, 64), (2, 256, 256, 128, 64, 64), (2, 64, 64, 32, 32, 128), (2, 32, 128, 32, 64, 64),
+                # 48- and 96-column wave tiles (three and six MFMA tile columns per wave)
+                (2, 256, 192, 128, 96, 64), (2, 128, 96, 64, 48, 128), (2, 32, 48, 32, 48, 64), (2, 128, 192, 32, 96, 128),
+                (2, 256, 96, 64, 96, 64)]
 
 
 # ---------------------------------------------------------------------------------------------
@@ -275,7 +278,8 @@ CONV_GEOMS_ODD = [(2, 20, 20, 3, 16, 7, 7, 2, 3), (1, 9, 11, 1, 8, 5, 5, 2, 0), 
 
 
 @pytest.mark.parametrize("cfg", [(2, 128, 128, 64, 64, 64), (2, 64, 64, 32, 32, 64), (2, 256, 64, 64, 32, 64),
-                                 (2, 128, 64, 64, 32, 128), (2, 256, 256, 128, 64, 64), (2, 64, 128, 32, 64, 64)])
+                                 (2, 128, 64, 64, 32, 128), (2, 256, 256, 128, 64, 64), (2, 64, 128, 32, 64, 64),
+                                 (2, 128, 96, 64, 48, 128), (2, 64, 192, 32, 96, 64)])
 def test_conv_f16_vs_oracle(cfg):
     lib = load(b16.kernel_library("gemm", *cfg))
     for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS + CONV_GEOMS_ODD:

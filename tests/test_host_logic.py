@@ -22,8 +22,8 @@ from MI355X_FP32 import profile_MI355X_FP32 as p32
 from MI355X_FP32 import MI355X_FP32_gemm as g32
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-N_FP16_CONFIGS = 106   # points of the FP16 template space (tile x wave tile x BLOCK_K) that fit LDS and registers
-N_FP16_SPLITK = 106    # every point also has a split-K variant
+N_FP16_CONFIGS = 159   # points of the FP16 template space (tile x wave tile x BLOCK_K) that fit LDS and registers
+N_FP16_SPLITK = 159    # every point also has a split-K variant
 
 
 # ---- enumeration ----------------------------------------------------------------------------------
