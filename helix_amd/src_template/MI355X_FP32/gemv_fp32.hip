@@ -44,7 +44,10 @@
 #define GEMV_KU16 1
 #endif
 #ifndef X_LDS_BYTES
-#define X_LDS_BYTES 65536   // LDS budget for the staged activations of one workgroup
+#define X_LDS_BYTES 65536   // staged activations of one workgroup of WAVES_PER_BLOCK waves (two workgroups share a CU)
+#endif
+#ifndef X_LDS_BYTES_WIDE
+#define X_LDS_BYTES_WIDE 131072   // ... of one workgroup of twice as many waves, alone on its CU: same waves per CU
 #endif
 #ifndef TARGET_WAVES
 #define TARGET_WAVES 2048   // waves a launch aims for: 256 compute units x 8
@@ -128,8 +131,11 @@ struct Reduce {
     }
 };
 
-template <int MT, int ROWS, int KU>
-__global__ __launch_bounds__(64 * WPB) void helix_gemv_f32_kernel(const Params p) {
+// WAVES: waves per workgroup.  WAVES_PER_BLOCK when the staged activations leave room for two workgroups per
+// CU, twice that when they need more than half of the LDS, so that a long K costs neither occupancy nor a
+// K partition with its second kernel.
+template <int MT, int ROWS, int KU, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void helix_gemv_f32_kernel(const Params p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     elem_t* xs = (elem_t*)smem;                      // [MT][kchunk] activations of this K range
 
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(64 * WPB) void helix_gemv_f32_kernel(const Params p
     constexpr int TRIP = KU * KSTEP;                 // K extent of one trip: KU*ROWS loads per lane
 
     // ---- this wave's run of weight rows -----------------------------------------------------------------
-    const int row_first = (blockIdx.x * WPB + wave) * p.rows_per_wave;
+    const int row_first = (blockIdx.x * WAVES + wave) * p.rows_per_wave;
     const int row_last = (row_first + p.rows_per_wave) < p.N ? (row_first + p.rows_per_wave) : p.N;
 
     const elem_t* wrow[ROWS];
@@ -175,7 +181,7 @@ __global__ __launch_bounds__(64 * WPB) void helix_gemv_f32_kernel(const Params p
     {
         const int chunks_per_row = kchunk / VEC;
         const int total = MT * chunks_per_row;
-        for (int c = tid; c < total; c += 64 * WPB) {
+        for (int c = tid; c < total; c += 64 * WAVES) {
             const int m = c / chunks_per_row, kc = (c % chunks_per_row) * VEC;
             intx4 v = {0, 0, 0, 0};
             if (m0 + m < p.M && k_begin + kc < k_end) v = *(const intx4*)(p.A + (size_t)(m0 + m) * p.lda + k_begin + kc);
@@ -311,11 +317,11 @@ inline const char* info_json() {
 
 constexpr int mtile_of(int M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
-// K partitioning: enough ranges that M_TILE activation rows of one range fit X_LDS_BYTES, at least SPLIT_K
+// K partitioning: enough ranges that M_TILE activation rows of one range fit X_LDS_BYTES_WIDE, at least SPLIT_K
 inline void k_partition(int M, int K, int* kchunk, int* ksplit) {
     const int mt = mtile_of(M);
     const int steps = (K + KSTEP - 1) / KSTEP;
-    int max_steps = X_LDS_BYTES / (mt * KSTEP * 4);
+    int max_steps = X_LDS_BYTES_WIDE / (mt * KSTEP * 4);
     if (max_steps < 1) max_steps = 1;
     int split = (steps + max_steps - 1) / max_steps;
     if (split < SPLITK) split = SPLITK;
@@ -336,20 +342,26 @@ inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce
     *lda = K; *ldb = K; *ldc = N;
 }
 
+template <int MT, int ROWS, int KU, int WAVES>
+inline int launch_waves(Params p, int lds, hipStream_t s) {
+    const int waves = (p.N + p.rows_per_wave - 1) / p.rows_per_wave;
+    static int attr_rc = (int)hipFuncSetAttribute((const void*)helix_gemv_f32_kernel<MT, ROWS, KU, WAVES>,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (attr_rc) return attr_rc;
+    dim3 grid((waves + WAVES - 1) / WAVES, (p.M + MT - 1) / MT, p.ksplit), block(64 * WAVES);
+    hipLaunchKernelGGL((helix_gemv_f32_kernel<MT, ROWS, KU, WAVES>), grid, block, lds, s, p);
+    return (int)hipGetLastError();
+}
+
 template <int MT, int ROWS, int KU>
 inline int launch_cfg(Params p, hipStream_t s) {
     // consecutive rows per wave: a multiple of ROWS that brings the launch near TARGET_WAVES waves
     long long want = ((long long)p.N * p.ksplit + TARGET_WAVES - 1) / TARGET_WAVES;
     if (want < 1) want = 1;
     p.rows_per_wave = (int)((want + ROWS - 1) / ROWS) * ROWS;
-    const int waves = (p.N + p.rows_per_wave - 1) / p.rows_per_wave;
     const int lds = MT * p.kchunk * 4;
-    static int attr_rc = (int)hipFuncSetAttribute((const void*)helix_gemv_f32_kernel<MT, ROWS, KU>,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (attr_rc) return attr_rc;
-    dim3 grid((waves + WPB - 1) / WPB, (p.M + MT - 1) / MT, p.ksplit), block(64 * WPB);
-    hipLaunchKernelGGL((helix_gemv_f32_kernel<MT, ROWS, KU>), grid, block, lds, s, p);
-    return (int)hipGetLastError();
+    if (lds > X_LDS_BYTES) return launch_waves<MT, ROWS, KU, 2 * WPB>(p, lds, s);
+    return launch_waves<MT, ROWS, KU, WPB>(p, lds, s);
 }
 
 inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc, void* ws,
