@@ -5,7 +5,7 @@ import os
 
 from utils.get_benchmark_shape_list import get_cnn_opset_shape_List
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP16.MI355X_FP16_conv import get_MI355X_FP16_conv_Helix_result
+from MI355X_FP16.MI355X_FP16_conv import get_MI355X_FP16_conv_Helix_result, get_MI355X_FP16_conv_miopen_result
 
 root_path = os.getcwd()
 
@@ -30,6 +30,20 @@ def MI355X_FP16_Helix_model_level_CNN_benchmark(backend="hip"):
     print(f'AlexNet: {helix_AlexNet_cost:.2f} ms, ResNet: {helix_ResNet_cost:.2f} ms, GoogleNet: {helix_GoogleNet_cost:.2f} ms')
 
 
+def MI355X_FP16_miopen_model_level_CNN_benchmark():
+    """Mirrors Ampere_FP16_cudnn_model_level_CNN_benchmark (benchmark_Ampere_FP16_model_level_CNN.py)."""
+    totals = []
+    for shape_list in get_cnn_opset_shape_List():
+        total, memo = 0, {}
+        for shape in shape_list:
+            if shape not in memo:
+                memo[shape], _ = get_MI355X_FP16_conv_miopen_result(*shape)
+            total += memo[shape]
+        totals.append(total)
+    print(f'AlexNet: {totals[0]:.2f} ms, ResNet: {totals[1]:.2f} ms, GoogleNet: {totals[2]:.2f} ms')
+
+
 if __name__ == "__main__":
 
     MI355X_FP16_Helix_model_level_CNN_benchmark(backend="hip")
+    MI355X_FP16_miopen_model_level_CNN_benchmark()

@@ -151,12 +151,19 @@ def build_jobs():
     jobs.append(compile_job("gemv"))
     jobs.append(compile_job("gemv_splitK"))
     jobs.append(rocblas_job())
+    jobs.append(miopen_job())
     return jobs
 
 
 def rocblas_job():
     """The vendor comparator, like the reference's `compile_kernel("cublas_f16")` (build_Ampere_FP16.py:72-76)."""
     return (f"{SRC_ROOT}/MI355X_FP16/rocblas_f16.hip", kernel_library("rocblas_f16"), {}, "-lrocblas")
+
+
+def miopen_job():
+    """The vendor convolution comparator, like the reference's `compile_kernel("cudnn_fp16")`
+    (build_Ampere_FP16.py)."""
+    return (f"{SRC_ROOT}/MI355X_FP16/miopen_f16.hip", kernel_library("miopen_f16"), {}, "-lMIOpen")
 
 
 def build_rocblas_FP16_gemm_kernel():

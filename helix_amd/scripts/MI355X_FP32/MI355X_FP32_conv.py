@@ -6,7 +6,7 @@ import math
 import os
 
 from utils.helix_runtime import load
-from MI355X_FP32.build_MI355X_FP32 import library_for_key
+from MI355X_FP32.build_MI355X_FP32 import library_for_key, kernel_library
 from MI355X_FP32.MI355X_FP32_gemm import config_cost, extra_points
 
 root_path = os.getcwd()
@@ -39,3 +39,15 @@ def get_MI355X_FP32_conv_Helix_result(prof_dict, batch, input_channel, H, W, out
     tflops = 2 * M * N * K / 1e9 / cost
 
     return cost, tflops
+
+
+def get_MI355X_FP32_conv_miopen_result(batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
+    """The vendor library on the same problem and layouts (miopenConvolutionForward with the algorithm MIOpen's own
+    search finds fastest), timed the same way.  Mirrors get_Ampere_FP32_conv_cudnn_result (Ampere_FP32_conv.py)."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    N = output_channel
+    K = input_channel * kH * kW
+    lib = load(kernel_library("miopen_f32"))
+    _, avg, _ = lib.bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad, warmup=10, iters=10)
+    cost = avg * 1e3
+    return cost, 2 * M * N * K / 1e9 / cost

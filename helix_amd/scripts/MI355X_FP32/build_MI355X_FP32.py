@@ -96,12 +96,18 @@ def build_jobs():
     jobs.append(compile_kernel("gemv_fp32"))
     jobs.append(compile_kernel("gemv_fp32_splitK"))
     jobs.append(rocblas_job())
+    jobs.append(miopen_job())
     return jobs
 
 
 def rocblas_job():
     """The vendor comparator, like the reference's cublas_f32 (build_Ampere_FP32.py:59-61)."""
     return (f"{SRC_ROOT}/MI355X_FP32/rocblas_f32.hip", kernel_library("rocblas_f32"), {}, "-lrocblas")
+
+
+def miopen_job():
+    """The vendor convolution comparator, like the reference's cudnn_fp32 (build_Ampere_FP32.py)."""
+    return (f"{SRC_ROOT}/MI355X_FP32/miopen_f32.hip", kernel_library("miopen_f32"), {}, "-lMIOpen")
 
 
 def build_Helix_MI355X_FP32_gemm_kernel():

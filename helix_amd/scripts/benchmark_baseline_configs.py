@@ -1,4 +1,4 @@
-"""python3 benchmark_baseline_configs.py -c {square,gemv,conv,bert,all} -b <backend> [--oracle] [--no-tiles] [--json]
+"""python3 benchmark_baseline_configs.py -c {square,gemv,conv,bert,all} -b <backend> [--oracle] [--no-tiles] [--vendor] [--json]
 
 The measured configurations of this backend, each against the roofline that bounds it:
   square  M = N = K in {1024, 2048, 4096, 8192}                              (MFMA peak)
@@ -94,7 +94,9 @@ def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
     return rows
 
 
-def conv_rows(be, prof_dict):
+def conv_rows(be, prof_dict, vendor=False):
+    """vendor=True adds MIOpen's time on the same layer (the comparator library)."""
+    miopen = load(be.build.kernel_library("miopen_f32" if be.fp32 else "miopen_f16")) if vendor else None
     rows = []
     for shp in S.get_baseline_conv_shape_list():
         b, ic, h, w, oc, kh, kw, st, pd = shp
@@ -106,6 +108,8 @@ def conv_rows(be, prof_dict):
                      "TFLOP/s": round(tflops, 2), "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4),
                      "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / (ms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
+        if miopen is not None:
+            rows[-1]["miopen_us"] = round(miopen.bench_conv(*shp, warmup=10, iters=10)[1] * 1e6, 2)
     return rows
 
 
@@ -130,7 +134,7 @@ def bert_rows(be, prof_dict):
 SECTIONS = {"square": square_rows, "gemv": gemv_rows, "conv": conv_rows, "bert": bert_rows}
 
 
-def run(backend, configs, oracle=False, tiles=True):
+def run(backend, configs, oracle=False, tiles=True, vendor=False):
     be = Backend(backend)
     prof_dict = be.prof_dict()
     out = {}
@@ -139,6 +143,8 @@ def run(backend, configs, oracle=False, tiles=True):
             out[name] = square_rows(be, prof_dict, oracle)
         elif name == "gemv":
             out[name] = gemv_rows(be, prof_dict, tiles=tiles)
+        elif name == "conv":
+            out[name] = conv_rows(be, prof_dict, vendor=vendor)
         else:
             out[name] = SECTIONS[name](be, prof_dict)
     return out
@@ -150,11 +156,12 @@ if __name__ == "__main__":
     parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default="MI355X_FP16")
     parser.add_argument("--oracle", action="store_true", help="also run the exhaustive search on the square shapes")
     parser.add_argument("--no-tiles", action="store_true", help="gemv: time the GEMV library only")
+    parser.add_argument("--vendor", action="store_true", help="conv: add MIOpen's time per layer")
     parser.add_argument("--json", action="store_true", help="one JSON object instead of the table")
     args = parser.parse_args()
 
     result = run(args.backend, list(SECTIONS) if args.config == "all" else [args.config], args.oracle,
-                 tiles=not args.no_tiles)
+                 tiles=not args.no_tiles, vendor=args.vendor)
     if args.json:
         print(json.dumps(result))
     else:

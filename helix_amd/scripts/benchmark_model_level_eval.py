@@ -12,13 +12,15 @@ func_dict = {
     ('CNN', 'MI355X_FP32', 'Helix'): ('MI355X_FP32.benchmark_MI355X_FP32_model_level_CNN', 'MI355X_FP32_Helix_model_level_CNN_benchmark'),
     ('LLM', 'MI355X_FP16', 'rocblas'): ('MI355X_FP16.benchmark_MI355X_FP16_model_level_LLM', 'MI355X_FP16_rocblas_model_level_LLM_benchmark'),
     ('LLM', 'MI355X_FP32', 'rocblas'): ('MI355X_FP32.benchmark_MI355X_FP32_model_level_LLM', 'MI355X_FP32_rocblas_model_level_LLM_benchmark'),
+    ('CNN', 'MI355X_FP16', 'miopen'): ('MI355X_FP16.benchmark_MI355X_FP16_model_level_CNN', 'MI355X_FP16_miopen_model_level_CNN_benchmark'),
+    ('CNN', 'MI355X_FP32', 'miopen'): ('MI355X_FP32.benchmark_MI355X_FP32_model_level_CNN', 'MI355X_FP32_miopen_model_level_CNN_benchmark'),
 }
 
 if __name__ == "__main__":
     parser = argparse.ArgumentParser(description="Benchmark Model level performance")
     parser.add_argument("-m", "--model", type=str, choices=['LLM', 'CNN'], default='LLM', help="model name")
     parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default='MI355X_FP16', help="backend")
-    parser.add_argument("-s", "--system", type=str, choices=['Helix', 'rocblas'], default='Helix', help="system")
+    parser.add_argument("-s", "--system", type=str, choices=['Helix', 'rocblas', 'miopen'], default='Helix', help="system")
     args = parser.parse_args()
 
     if (args.model, args.backend, args.system) in func_dict.keys():

@@ -366,6 +366,27 @@ def test_rocblas_comparators_vs_oracle():
     assert 0 < mn <= avg <= mx
 
 
+def test_miopen_comparators_vs_oracle():
+    """The MIOpen comparator libraries describe the templates' layouts (NHWC activations, [OC][kH][kW][IC] weights)
+    to the vendor library; a wrong dimension order or layout fails here, before any benchmark prints a vendor
+    column.  FP32 tolerance 1e-4: the vendor's algorithm (picked by its own search) may not sum in k order."""
+    geoms = [(2, 14, 14, 16, 24, 3, 3, 1, 1), (2, 15, 13, 8, 8, 3, 3, 2, 1), (3, 8, 8, 32, 16, 1, 1, 2, 0),
+             (2, 9, 9, 64, 64, 3, 3, 1, 1)]
+    for lib, dtype, tol, cast in ((load(b16.kernel_library("miopen_f16")), torch.float16, TOL16, np.float16),
+                                  (load(b32.kernel_library("miopen_f32")), torch.float32, 1e-4, np.float32)):
+        assert lib.info()["family"] == "miopen"
+        for (batch, H, W, IC, OC, kH, kW, stride, pad) in geoms:
+            x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW)
+            x, w = x.astype(cast), w.astype(cast)
+            got = run_conv(lib, x, w, stride, pad, dtype)
+            want = O.conv2d_nhwc(x, w, stride, pad)
+            assert got.shape == want.shape
+            assert not np.isnan(got).any(), (dtype, batch, H, W, IC, OC, kH, kW, stride, pad)
+            assert normwise(got, want) < tol, (dtype, batch, H, W, IC, OC, kH, kW, stride, pad)
+        mn, avg, mx = lib.bench_conv(2, 16, 14, 14, 24, 3, 3, 1, 1, warmup=2, iters=3)
+        assert 0 < mn <= avg <= mx
+
+
 # ---------------------------------------------------------------------------------------------
 # FP32
 # ---------------------------------------------------------------------------------------------
