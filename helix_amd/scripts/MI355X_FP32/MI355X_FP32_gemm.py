@@ -13,6 +13,10 @@ root_path = os.getcwd()
 
 HBM_SUSTAINED_FRACTION = 0.8
 GEMV_LAUNCH_FLOOR_S = 3.4e-6
+# the weight-streaming kernels pass over the weights once per 16 activation rows: beyond one pass a tile kernel,
+# which reads them once per BLOCK_ROWS rows, is the better streamer, and the per-round share the model assumes
+# for them no longer holds (measured: 661 x 768 x 3072 FP32, 103 us against 27 us)
+GEMV_MAX_ROWS = 16
 GEMV_SPLITK_EXTRA_S = 2e-6        # the K-partitioned library's reduction pass on a problem too small to need it
 # a further round of tiles costs what the two-round profile shows beyond one round, but never less than this
 # share of a lone round: the profiled problems sit in the caches, long ones do not
@@ -20,6 +24,23 @@ LATER_ROUND_MIN_SHARE = 0.5
 # rate at which the compute units take A and B tiles in (bytes of M*N*K*4*(1/BM + 1/BN) per second): what the
 # small-tile configurations reach on 2048^3 ... 8192^3
 OPERAND_BYTES_PER_S = 6.5e12
+
+
+SPLITK_MAX, SPLITK_MAX_TILES, SPLITK_MIN_KTILES = 8, 192, 8   # as in src_template/MI355X_FP32/sgemm.hip
+SPLITK_REDUCE_LAUNCH_S = 4e-6   # the reduction kernel of a K-partitioned launch
+
+
+def split_factor(k, M, N, K):
+    """K partitions the SGEMM libraries use for this problem (same rule as their host side): only when the
+    tiles alone leave compute units idle, as many as bring the launch to about one workgroup per compute unit,
+    at most SPLITK_MAX, at least SPLITK_MIN_KTILES K tiles per partition."""
+    if k[2] == 0:
+        return 1
+    tiles = math.ceil(M / k[0]) * math.ceil(N / k[1])
+    ktiles = math.ceil(K / k[2])
+    if tiles <= 0 or tiles >= SPLITK_MAX_TILES:
+        return 1
+    return max(min(math.ceil(256 / tiles), SPLITK_MAX, ktiles // SPLITK_MIN_KTILES), 1)
 
 
 def _line(x0, y0, x1, y1, x):
@@ -37,21 +58,28 @@ def config_cost(k, v, M, N, K, points=None):
     and each further round the line through the two-round increments."""
     if k[2] == 0:
         small, big = (M, N) if M <= N else (N, M)
+        if small > GEMV_MAX_ROWS:
+            return float("inf")
         num_block = math.ceil(small / k[0]) * math.ceil(big / k[1])
         cost = max(num_block / NUM_CU * v * max(K, 256) / GEMV_PROFILE_K, GEMV_LAUNCH_FLOOR_S)
         return cost + (GEMV_SPLITK_EXTRA_S if k[5] == 1 else 0.0)
     tiles_m, tiles_n = math.ceil(M / k[0]), math.ceil(N / k[1])
-    w = math.ceil(tiles_m * tiles_n / NUM_CU)
+    splits = split_factor(k, M, N, K)
+    w = math.ceil(tiles_m * tiles_n * splits / NUM_CU)
     hbm_floor = gemm_bytes(M, N, K, 4) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S)
+    # K a workgroup walks, in whole BK steps
+    k_walk = math.ceil(math.ceil(K / k[2]) / splits) * k[2]
+    # the partial sums are written and read back by a second kernel
+    reduce = 0.0 if splits == 1 else (SPLITK_REDUCE_LAUNCH_S +
+                                      (splits + 1) * M * N * 4 / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
     if points is None or not _finite(v, *points):
-        return max(w * v * max(K, 32) / PROFILE_K, hbm_floor)
+        return max(w * v * max(k_walk, 32) / PROFILE_K + reduce, hbm_floor)
     short, two, short_two = points
-    k_walk = math.ceil(K / k[2]) * k[2]
     first = max(_line(PROFILE_K_SHORT, short, PROFILE_K, v, k_walk), 0.25 * short)
     later = _line(PROFILE_K_SHORT, short_two - short, PROFILE_K, two - v, k_walk)
     later = min(max(later, LATER_ROUND_MIN_SHARE * first), first)
     operand_floor = 4.0 * tiles_m * k[0] * tiles_n * k[1] * K * (1 / k[0] + 1 / k[1]) / OPERAND_BYTES_PER_S
-    return max(first + (w - 1) * later, hbm_floor, operand_floor)
+    return max(first + (w - 1) * later + reduce, hbm_floor, operand_floor)
 
 
 def extra_points(prof_dict, k):

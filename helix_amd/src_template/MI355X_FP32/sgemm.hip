@@ -12,6 +12,11 @@
 //
 // Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N.
 //
+// K partitions: a problem whose tiles alone would leave compute units idle (fewer than 192 tiles) and whose K is
+// long is split along K over blockIdx.y, up to 8 ways; partial sums go to the caller's workspace
+// (helix_workspace_bytes) and a second kernel adds them in partition order.  Without the workspace the
+// problem runs unpartitioned.  The reference's FP32 template has no K partition.
+//
 // LDS layout: A stage is [BK][BM + 32] floats, B stage [BK][BN + 32]; a fragment read takes lanes 0-31
 // from row k and lanes 32-63 from row k+1, and the 32-float row padding puts the two half-waves on
 // different halves of the 64 banks.  In CONV mode operands arrive K-contiguous and are written
@@ -83,6 +88,9 @@ struct Params {
     int M, N, K, lda, ldb, ldc;
     int tiles_m, tiles_n;
     unsigned a_bytes;
+    float* ws;       // splits > 1: [splits][M][N] partial sums
+    int splits;      // K partitions of this launch (grid.y)
+    int k_per;       // K extent of one partition, a multiple of BK
     ConvGeom g;
 };
 
@@ -122,6 +130,10 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     const int tile_n = (pid % group_tiles) / gsize;
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
+    // K range of this workgroup
+    const int k_lo = (int)blockIdx.y * p.k_per;
+    const int k_hi = (k_lo + p.k_per) < p.K ? (k_lo + p.k_per) : p.K;
+
     constexpr int NA = CONV ? AC_ITERS : A_ITERS;
     constexpr int NB = CONV ? BC_ITERS : B_ITERS;
     floatx4 stage_a[NA], stage_b[NB];
@@ -146,9 +158,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
         if (!CONV) {
             // rows k0.. of A^T (K x M) starting at column m0; whole rows are inside the buffer, rows >= K are not
             __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + (size_t)k0 * p.lda + m0,
-                                                  (unsigned)(((size_t)(p.K - k0) * p.lda - m0) * 4));
+                                                  (unsigned)(((size_t)(k_hi - k0) * p.lda - m0) * 4));
             __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)k0 * p.ldb + n0,
-                                                  (unsigned)(((size_t)(p.K - k0) * p.ldb - n0) * 4));
+                                                  (unsigned)(((size_t)(k_hi - k0) * p.ldb - n0) * 4));
 #pragma unroll
             for (int i = 0; i < NA; i++) {
                 const int c = tid + i * NTHREADS;
@@ -163,7 +175,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
             __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, p.a_bytes);
             const int kc = tid % K_CPR;
             const int k = k0 + kc * 4;
-            const bool dead = k >= p.K;
+            const bool dead = k >= k_hi;
             const int t = p.g.by_IC.div(k);
             const int c = k - t * p.g.IC;
             const int kh = p.g.by_kW.div(t);
@@ -229,15 +241,17 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     const int a_rd = fk * LDA_S + wave_m * WAVE_M + frow;
     const int b_rd = A_STAGE + fk * LDB_S + wave_n * WAVE_N + frow;
 
-    const int ktiles = (p.K + BK - 1) / BK;
-    load_global(0);
-    store_lds(0);
+    const int ktiles = (k_hi - k_lo + BK - 1) / BK;
+    if (ktiles > 0) {
+        load_global(k_lo);
+        store_lds(0);
+    }
     __syncthreads();
 
     for (int kt = 0; kt < ktiles; kt++) {
         const int cur = kt & 1;
         const bool more = (kt + 1 < ktiles);
-        if (more) load_global((kt + 1) * BK);
+        if (more) load_global(k_lo + (kt + 1) * BK);
 
         const float* sb = smem + cur * STAGE;
 #pragma unroll
@@ -268,9 +282,23 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 #pragma unroll
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wave_m * WAVE_M + i * 32 + (v / 4) * 8 + row_l + (v % 4);
-                if (row < p.M && col < p.N) p.C[(size_t)row * p.ldc + col] = acc[i][j][v];
+                if (row < p.M && col < p.N) {
+                    if (p.splits > 1) p.ws[((size_t)blockIdx.y * p.M + row) * p.N + col] = acc[i][j][v];
+                    else p.C[(size_t)row * p.ldc + col] = acc[i][j][v];
+                }
             }
         }
+    }
+}
+
+// Sums the K partitions in a fixed order (deterministic).
+__global__ void helix_sgemm_splitk_reduce_kernel(const float* ws, float* C, int M, int N, int ldc, int splits) {
+    const size_t total = (size_t)M * N;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        float s = 0.f;
+        for (int k = 0; k < splits; k++) s += ws[(size_t)k * total + idx];
+        C[(idx / N) * ldc + idx % N] = s;
     }
 }
 
@@ -289,7 +317,7 @@ inline const char* info_json() {
         snprintf(buf, sizeof(buf),
                  "{\"family\": \"sgemm_f32\", \"arch\": \"gfx950\", \"mfma\": \"v_mfma_f32_32x32x2_f32\", "
                  "\"lds_stages\": 2, \"block_rows\": %d, \"block_cols\": %d, \"wave_rows\": %d, \"wave_cols\": %d, "
-                 "\"block_k\": %d, \"split_k\": 1, \"threads\": %d, \"lds_bytes\": %d, "
+                 "\"block_k\": %d, \"split_k\": \"up to 8 K partitions when the tiles leave compute units idle and the caller passes the workspace\", \"threads\": %d, \"lds_bytes\": %d, "
                  "\"layout_a\": \"K x M row-major f32 (A transposed)\", \"layout_b\": \"K x N row-major f32\", "
                  "\"layout_c\": \"M x N row-major f32\", \"accumulate\": \"f32\", "
                  "\"k_multiple\": 1, \"ld_multiple\": 4, \"conv\": \"NHWC x [OC][kH][kW][IC]; implicit GEMM when IC %% 4 == 0, else column buffer in the workspace\"}",
@@ -299,7 +327,28 @@ inline const char* info_json() {
     return buf;
 }
 
-inline size_t workspace_bytes(int, int, int) { return 0; }
+// K partitions for an M x N x K problem: only when the tiles alone leave compute units idle (fewer than
+// SPLITK_MAX_TILES of them), as many as bring the launch to about one workgroup per compute unit, at most
+// SPLITK_MAX, and never so many that a partition walks fewer than SPLITK_MIN_KTILES K tiles.  The reference's
+// FP32 template has no K partition (src_template/Ampere_FP32/sgemm.cu); its FP16 one is 2-way
+// (gemm_splitK.cu:124-129).
+constexpr int SPLITK_MAX = 8, SPLITK_MAX_TILES = 192, SPLITK_MIN_KTILES = 8;
+
+inline int split_factor(long long M, long long N, long long K) {
+    const long long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+    const long long ktiles = (K + BK - 1) / BK;
+    if (tiles <= 0 || tiles >= SPLITK_MAX_TILES) return 1;
+    long long s = (256 + tiles - 1) / tiles;
+    if (s > SPLITK_MAX) s = SPLITK_MAX;
+    if (s > ktiles / SPLITK_MIN_KTILES) s = ktiles / SPLITK_MIN_KTILES;
+    return s < 1 ? 1 : (int)s;
+}
+
+// Partial sums of the K partitions; a caller that passes less runs the problem unpartitioned.
+inline size_t workspace_bytes(int M, int N, int K) {
+    const int s = split_factor(M, N, K);
+    return s > 1 ? (size_t)s * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
 
 inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce, int* lda, int* ldb, int* ldc) {
     const int Mp = (M + 3) / 4 * 4, Np = (N + 3) / 4 * 4;
@@ -308,18 +357,34 @@ inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce
 }
 
 template <bool CONV>
-inline int launch(const Params& p, hipStream_t s) {
+inline int launch(Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
     static int rc = (int)hipFuncSetAttribute((const void*)helix_sgemm_f32_kernel<CONV>,
                                              hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES);
     if (rc) return rc;
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
-    hipLaunchKernelGGL(helix_sgemm_f32_kernel<CONV>, dim3((unsigned)ntiles), dim3(NTHREADS), LDS_BYTES, s, p);
-    return (int)hipGetLastError();
+    p.splits = split_factor(p.M, p.N, p.K);
+    if (p.splits > 1 && (!ws || ((uintptr_t)ws & 3) || ws_bytes < workspace_bytes(p.M, p.N, p.K))) p.splits = 1;
+    const int ktiles = (p.K + BK - 1) / BK;
+    p.k_per = ((ktiles + p.splits - 1) / p.splits) * BK;
+    p.ws = (float*)ws;
+    hipLaunchKernelGGL(helix_sgemm_f32_kernel<CONV>, dim3((unsigned)ntiles, (unsigned)p.splits), dim3(NTHREADS),
+                       LDS_BYTES, s, p);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    if (p.splits > 1) {
+        const size_t total = (size_t)p.M * p.N;
+        int blocks = (int)((total + 255) / 256);
+        if (blocks > 8192) blocks = 8192;
+        hipLaunchKernelGGL(helix_sgemm_splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, (const float*)ws, p.C, p.M,
+                           p.N, p.ldc, p.splits);
+        e = hipGetLastError();
+    }
+    return (int)e;
 }
 
-inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc, void*, size_t,
-                hipStream_t s) {
+inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc, void* ws,
+                size_t ws_bytes, hipStream_t s) {
     if (lda % 4 != 0 || ldb % 4 != 0) return HELIX_ERR_INVALID_VALUE;  // 16-byte loads along M and N
     if (lda < M || ldb < N || ldc < N) return HELIX_ERR_INVALID_VALUE;
     if (((uintptr_t)A & 15) || ((uintptr_t)B & 15) || ((uintptr_t)C & 3)) return HELIX_ERR_INVALID_VALUE;
@@ -332,17 +397,19 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     p.A = (const float*)A; p.B = (const float*)B; p.C = (float*)C;
     p.M = M; p.N = N; p.K = K; p.lda = lda; p.ldb = ldb; p.ldc = ldc;
     p.tiles_m = (M + BM - 1) / BM; p.tiles_n = (N + BN - 1) / BN;
-    return launch<false>(p, s);
+    return launch<false>(p, ws, ws_bytes, s);
 }
 
 // Convolutions whose channel count is not a multiple of 4 go through a column buffer (K x M, the A layout of
 // this template) and transposed weights (K x N) in the workspace, then through the GEMM above.
 inline size_t conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad) {
-    if (IC % 4 == 0) return 0;
     const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
     const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
+    if (M > 0x7fffffffLL || K > 0x7fffffffLL) return 0;
+    if (IC % 4 == 0) return workspace_bytes((int)M, OC, (int)K);
     const long long Mp = (M + 3) / 4 * 4, Np = (OC + 3) / 4 * 4;
-    return helix_im2col::align256((size_t)K * Mp * 4) + helix_im2col::align256((size_t)K * Np * 4);
+    return helix_im2col::align256((size_t)K * Mp * 4) + helix_im2col::align256((size_t)K * Np * 4) +
+           workspace_bytes((int)M, OC, (int)K);
 }
 
 inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
@@ -362,7 +429,8 @@ inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int
                        dim3(256), 0, s, (const float*)w, wt, OC, (int)K, Np);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    return gemm(col, wt, y, (int)M, OC, (int)K, Mp, Np, OC, nullptr, 0, s);
+    const size_t used = col_bytes + helix_im2col::align256((size_t)K * Np * 4);
+    return gemm(col, wt, y, (int)M, OC, (int)K, Mp, Np, OC, (unsigned char*)ws + used, ws_bytes - used, s);
 }
 
 inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
@@ -382,7 +450,7 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
     p.a_bytes = (unsigned)xbytes;
     p.g = ConvGeom{H, W, IC, OH, OW, kW, stride, pad, (int)M,
                    helix_fastdiv::make(OW), helix_fastdiv::make(OH), helix_fastdiv::make(IC), helix_fastdiv::make(kW)};
-    return launch<true>(p, s);
+    return launch<true>(p, ws, ws_bytes, s);
 }
 
 }  // namespace tpl

@@ -58,8 +58,9 @@ def run_gemm_f16(lib, A, B, ldpad=0):
     return dC.cpu().numpy()
 
 
-def run_sgemm_f32(lib, A, B):
-    """A (M,K) f32, B (K,N) f32 -> C (M,N) f32 through helix_gemm (device layout: A as K x M)."""
+def run_sgemm_f32(lib, A, B, workspace=True):
+    """A (M,K) f32, B (K,N) f32 -> C (M,N) f32 through helix_gemm (device layout: A as K x M).  With the
+    workspace the library asks for, few-tile problems are K-partitioned; without it they run unpartitioned."""
     M, K = A.shape
     N = B.shape[1]
     Mp, Np = (M + 3) // 4 * 4, (N + 3) // 4 * 4
@@ -69,7 +70,9 @@ def run_sgemm_f32(lib, A, B):
     Bp[:, :N] = B
     dA, dB = dev(At), dev(Bp)
     dC = torch.full((M, N), float("nan"), dtype=torch.float32, device="cuda:0")
-    lib.gemm(dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), M, N, K, Mp, Np, N, 0, 0,
+    wsb = lib.workspace_bytes(M, N, K) if workspace else 0
+    ws = torch.empty(max(wsb, 16), dtype=torch.uint8, device="cuda:0")
+    lib.gemm(dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), M, N, K, Mp, Np, N, ws.data_ptr() if wsb else 0, wsb,
              torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     return dC.cpu().numpy()
@@ -390,6 +393,33 @@ def test_miopen_comparators_vs_oracle():
 # ---------------------------------------------------------------------------------------------
 # FP32
 # ---------------------------------------------------------------------------------------------
+def test_sgemm_f32_k_partitions():
+    """Problems with few output tiles and a long K are partitioned along K when the caller passes the workspace
+    `helix_workspace_bytes` asks for (partial sums + fixed-order reduction), and run unpartitioned otherwise:
+    both agree with the oracle, and on integer-valued inputs both are exact."""
+    rng = np.random.default_rng(21)
+    for cfg in [(64, 64, 32, 32, 32), (128, 128, 16, 64, 64), (32, 32, 8, 32, 32)]:
+        lib = load(b32.sgemm_library(*cfg))
+        BM, BN, BK = cfg[:3]
+        for (M, N, K) in [(100, 96, 2048), (257, 129, 1000), (64, 64, 8 * BK * 8), (300, 200, 137), (33, 500, 4096)]:
+            tiles = -(-M // BM) * -(-N // BN)
+            ktiles = -(-K // BK)
+            want_splits = 1 if tiles >= 192 else max(min(-(-256 // tiles), 8, ktiles // 8), 1)
+            assert lib.workspace_bytes(M, N, K) == (want_splits * M * N * 4 if want_splits > 1 else 0), (cfg, M, N, K)
+            A = seeded_inputs.uniform_pm1((M, K), seeded_inputs.SEED_A)
+            B = seeded_inputs.uniform_pm1((K, N), seeded_inputs.SEED_B)
+            want = O.sgemm_seqk(A, B)
+            for workspace in (True, False):
+                got = run_sgemm_f32(lib, A, B, workspace)
+                assert not np.isnan(got).any(), (cfg, M, N, K, workspace)
+                assert normwise(got, want) < TOL32, (cfg, M, N, K, workspace)
+            Ai = rng.integers(-3, 4, (M, K)).astype(np.float32)
+            Bi = rng.integers(-3, 4, (K, N)).astype(np.float32)
+            exact = (Ai.astype(np.int64) @ Bi.astype(np.int64)).astype(np.float32)
+            assert np.array_equal(run_sgemm_f32(lib, Ai, Bi, True), exact), (cfg, M, N, K)
+            assert np.array_equal(run_sgemm_f32(lib, Ai, Bi, False), exact), (cfg, M, N, K)
+
+
 FP32_CONFIGS = [(128, 128, 16, 64, 64), (256, 128, 16, 128, 64), (32, 32, 8, 32, 32), (64, 256, 32, 32, 128),
                 (128, 64, 32, 64, 32)]
 
