@@ -26,21 +26,22 @@ LATER_ROUND_MIN_SHARE = 0.5
 OPERAND_BYTES_PER_S = 6.5e12
 
 
-SPLITK_MAX, SPLITK_MAX_TILES, SPLITK_MIN_KTILES = 8, 192, 8   # as in src_template/MI355X_FP32/sgemm.hip
+SPLITK_MAX, SPLITK_TARGET, SPLITK_MIN_K = 8, 768, 768   # as in src_template/MI355X_FP32/sgemm.hip
+SPLITK_MIN_K_FEW, SPLITK_FEW_TILES = 256, 128
 SPLITK_REDUCE_LAUNCH_S = 4e-6   # the reduction kernel of a K-partitioned launch
 
 
 def split_factor(k, M, N, K):
-    """K partitions the SGEMM libraries use for this problem (same rule as their host side): only when the
-    tiles alone leave compute units idle, as many as bring the launch to about one workgroup per compute unit,
-    at most SPLITK_MAX, at least SPLITK_MIN_KTILES K tiles per partition."""
+    """K partitions the SGEMM libraries use for this problem (same rule as their host side): when the tiles give
+    fewer than three quarters of SPLITK_TARGET workgroups, as many as reach the target, at most SPLITK_MAX, at
+    least SPLITK_MIN_K of K per partition (SPLITK_MIN_K_FEW when there are at most SPLITK_FEW_TILES tiles)."""
     if k[2] == 0:
         return 1
     tiles = math.ceil(M / k[0]) * math.ceil(N / k[1])
-    ktiles = math.ceil(K / k[2])
-    if tiles <= 0 or tiles >= SPLITK_MAX_TILES:
+    if tiles <= 0 or tiles >= SPLITK_TARGET * 3 // 4:
         return 1
-    return max(min(math.ceil(256 / tiles), SPLITK_MAX, ktiles // SPLITK_MIN_KTILES), 1)
+    min_k = SPLITK_MIN_K_FEW if tiles <= SPLITK_FEW_TILES else SPLITK_MIN_K
+    return max(min(math.ceil(SPLITK_TARGET / tiles), SPLITK_MAX, K // min_k), 1)
 
 
 def _line(x0, y0, x1, y1, x):

@@ -12,8 +12,8 @@
 //
 // Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N.
 //
-// K partitions: a problem whose tiles alone would leave compute units idle (fewer than 192 tiles) and whose K is
-// long is split along K over blockIdx.y, up to 8 ways; partial sums go to the caller's workspace
+// K partitions: a problem with fewer than 576 output tiles and a long K is split along K over blockIdx.y, up
+// to 8 ways (at least 768 of K each, 256 when there are at most 128 tiles); partial sums go to the caller's workspace
 // (helix_workspace_bytes) and a second kernel adds them in partition order.  Without the workspace the
 // problem runs unpartitioned.  The reference's FP32 template has no K partition.
 //
@@ -45,6 +45,9 @@
 #endif
 #ifndef GROUP_ROWS
 #define GROUP_ROWS 8
+#endif
+#ifndef SPLITK_TARGET_BLOCKS
+#define SPLITK_TARGET_BLOCKS 768   // workgroups a K-partitioned launch aims for: three per compute unit
 #endif
 
 namespace {
@@ -327,20 +330,23 @@ inline const char* info_json() {
     return buf;
 }
 
-// K partitions for an M x N x K problem: only when the tiles alone leave compute units idle (fewer than
-// SPLITK_MAX_TILES of them), as many as bring the launch to about one workgroup per compute unit, at most
-// SPLITK_MAX, and never so many that a partition walks fewer than SPLITK_MIN_KTILES K tiles.  The reference's
-// FP32 template has no K partition (src_template/Ampere_FP32/sgemm.cu); its FP16 one is 2-way
-// (gemm_splitK.cu:124-129).
-constexpr int SPLITK_MAX = 8, SPLITK_MAX_TILES = 192, SPLITK_MIN_KTILES = 8;
+// K partitions for an M x N x K problem: when the tiles alone give fewer than three quarters of SPLITK_TARGET
+// workgroups (three per compute unit: this kernel hides its LDS and global latencies across workgroups that share
+// a compute unit, and a launch of one to two rounds of tiles leaves most units with one), as many as reach
+// the target, at most SPLITK_MAX, and never so many that a partition walks less than SPLITK_MIN_K of K
+// (SPLITK_MIN_K_FEW when the tiles do not even cover half of the compute units).
+// Measured on 1521 x 768 x 2304: 83 us unpartitioned, 62 us three-way.  The reference's FP32 template has no K
+// partition (src_template/Ampere_FP32/sgemm.cu); its FP16 one is 2-way (gemm_splitK.cu:124-129).
+constexpr int SPLITK_MAX = 8, SPLITK_TARGET = SPLITK_TARGET_BLOCKS, SPLITK_MAX_TILES = SPLITK_TARGET * 3 / 4,
+              SPLITK_MIN_K = 768, SPLITK_MIN_K_FEW = 256, SPLITK_FEW_TILES = 128;
 
 inline int split_factor(long long M, long long N, long long K) {
     const long long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    const long long ktiles = (K + BK - 1) / BK;
     if (tiles <= 0 || tiles >= SPLITK_MAX_TILES) return 1;
-    long long s = (256 + tiles - 1) / tiles;
+    long long s = (SPLITK_TARGET + tiles - 1) / tiles;
     if (s > SPLITK_MAX) s = SPLITK_MAX;
-    if (s > ktiles / SPLITK_MIN_KTILES) s = ktiles / SPLITK_MIN_KTILES;
+    const long long min_k = tiles <= SPLITK_FEW_TILES ? SPLITK_MIN_K_FEW : SPLITK_MIN_K;
+    if (s > K / min_k) s = K / min_k;
     return s < 1 ? 1 : (int)s;
 }
 
