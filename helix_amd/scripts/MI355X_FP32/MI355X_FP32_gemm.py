@@ -18,9 +18,18 @@ GEMV_LAUNCH_FLOOR_S = 3.4e-6
 # for them no longer holds (measured: 661 x 768 x 3072 FP32, 103 us against 27 us)
 GEMV_MAX_ROWS = 16
 GEMV_SPLITK_EXTRA_S = 2e-6        # the K-partitioned library's reduction pass on a problem too small to need it
-# a further round of tiles costs what the two-round profile shows beyond one round, but never less than this
-# share of a lone round: the profiled problems sit in the caches, long ones do not
-LATER_ROUND_MIN_SHARE = 0.5
+# a further round of tiles costs what the two-round profile shows beyond one round, but never less than a share of
+# a lone round: the profiled problems sit in the caches, long ones do not.  The share grows with the K a workgroup
+# walks (workgroups sharing a compute unit overlap each other's latencies on short walks; on long ones they compete
+# for the caches): SHORT up to the profile K, LONG from four times that, linear in between.
+LATER_ROUND_MIN_SHARE_SHORT = 0.5
+LATER_ROUND_MIN_SHARE_LONG = 0.85
+
+
+def later_round_min_share(k_walk):
+    t = min(max((k_walk - PROFILE_K) / (3.0 * PROFILE_K), 0.0), 1.0)
+    return LATER_ROUND_MIN_SHARE_SHORT + (LATER_ROUND_MIN_SHARE_LONG - LATER_ROUND_MIN_SHARE_SHORT) * t
+
 # rate at which the compute units take A and B tiles in (bytes of M*N*K*4*(1/BM + 1/BN) per second): what the
 # small-tile configurations reach on 2048^3 ... 8192^3
 OPERAND_BYTES_PER_S = 6.5e12
@@ -78,7 +87,7 @@ def config_cost(k, v, M, N, K, points=None):
     short, two, short_two = points
     first = max(_line(PROFILE_K_SHORT, short, PROFILE_K, v, k_walk), 0.25 * short)
     later = _line(PROFILE_K_SHORT, short_two - short, PROFILE_K, two - v, k_walk)
-    later = min(max(later, LATER_ROUND_MIN_SHARE * first), first)
+    later = min(max(later, later_round_min_share(k_walk) * first), first)
     operand_floor = 4.0 * tiles_m * k[0] * tiles_n * k[1] * K * (1 / k[0] + 1 / k[1]) / OPERAND_BYTES_PER_S
     return max(first + (w - 1) * later + reduce, hbm_floor, operand_floor)
 

@@ -24,6 +24,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "helix_abi.h"
 #include "helix_im2col.h"
 #include "helix_fastdiv.h"
@@ -139,7 +141,9 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 
     constexpr int NA = CONV ? AC_ITERS : A_ITERS;
     constexpr int NB = CONV ? BC_ITERS : B_ITERS;
-    floatx4 stage_a[NA], stage_b[NB];
+    // two sets of staging registers: a K tile is requested two tiles ahead of its use, so that its loads have
+    // a whole tile of MFMAs plus the previous tile's LDS writes to land
+    floatx4 stage_a[2][NA], stage_b[2][NB];
 
     // CONV: per-row gather state
     int cv_img[NA], cv_ih[NA], cv_iw[NA];
@@ -157,7 +161,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
         }
     }
 
-    auto load_global = [&](int k0) {
+    auto load_global = [&](int k0, auto set_c) {
+        constexpr int SET = decltype(set_c)::value;
         if (!CONV) {
             // rows k0.. of A^T (K x M) starting at column m0; whole rows are inside the buffer, rows >= K are not
             __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + (size_t)k0 * p.lda + m0,
@@ -167,12 +172,12 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 #pragma unroll
             for (int i = 0; i < NA; i++) {
                 const int c = tid + i * NTHREADS;
-                stage_a[i] = buf_load16(ra, ((c / A_CPR) * p.lda + (c % A_CPR) * 4) * 4);
+                stage_a[SET][i] = buf_load16(ra, ((c / A_CPR) * p.lda + (c % A_CPR) * 4) * 4);
             }
 #pragma unroll
             for (int i = 0; i < NB; i++) {
                 const int c = tid + i * NTHREADS;
-                stage_b[i] = buf_load16(rb, ((c / B_CPR) * p.ldb + (c % B_CPR) * 4) * 4);
+                stage_b[SET][i] = buf_load16(rb, ((c / B_CPR) * p.ldb + (c % B_CPR) * 4) * 4);
             }
         } else {
             __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, p.a_bytes);
@@ -187,7 +192,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
             for (int i = 0; i < NA; i++) {
                 const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
                 const bool ok = !dead && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W;
-                stage_a[i] = buf_load16(ra, ok ? ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 4 : OOB);
+                stage_a[SET][i] = buf_load16(ra, ok ? ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 4 : OOB);
             }
             // weights: N x K row-major; rows >= N fall outside the buffer
             const int rows_b = (p.N - n0) < BN ? (p.N - n0) : BN;
@@ -195,24 +200,25 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 #pragma unroll
             for (int i = 0; i < NB; i++) {
                 const int n = (tid + i * NTHREADS) / K_CPR;
-                stage_b[i] = buf_load16(rb, dead ? OOB : (n * p.K + k) * 4);
+                stage_b[SET][i] = buf_load16(rb, dead ? OOB : (n * p.K + k) * 4);
             }
         }
     };
 
-    auto store_lds = [&](int stage) {
+    auto store_lds = [&](int stage, auto set_c) {
+        constexpr int SET = decltype(set_c)::value;
         float* sa = smem + stage * STAGE;
         float* sb = sa + A_STAGE;
         if (!CONV) {
 #pragma unroll
             for (int i = 0; i < NA; i++) {
                 const int c = tid + i * NTHREADS;
-                *(floatx4*)(sa + (c / A_CPR) * LDA_S + (c % A_CPR) * 4) = stage_a[i];
+                *(floatx4*)(sa + (c / A_CPR) * LDA_S + (c % A_CPR) * 4) = stage_a[SET][i];
             }
 #pragma unroll
             for (int i = 0; i < NB; i++) {
                 const int c = tid + i * NTHREADS;
-                *(floatx4*)(sb + (c / B_CPR) * LDB_S + (c % B_CPR) * 4) = stage_b[i];
+                *(floatx4*)(sb + (c / B_CPR) * LDB_S + (c % B_CPR) * 4) = stage_b[SET][i];
             }
         } else {
             const int kc = (tid % K_CPR) * 4;
@@ -220,13 +226,13 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
             for (int i = 0; i < NA; i++) {
                 const int m = (tid + i * NTHREADS) / K_CPR;
 #pragma unroll
-                for (int e = 0; e < 4; e++) sa[(kc + e) * LDA_S + m] = stage_a[i][e];
+                for (int e = 0; e < 4; e++) sa[(kc + e) * LDA_S + m] = stage_a[SET][i][e];
             }
 #pragma unroll
             for (int i = 0; i < NB; i++) {
                 const int n = (tid + i * NTHREADS) / K_CPR;
 #pragma unroll
-                for (int e = 0; e < 4; e++) sb[(kc + e) * LDB_S + n] = stage_b[i][e];
+                for (int e = 0; e < 4; e++) sb[(kc + e) * LDB_S + n] = stage_b[SET][i][e];
             }
         }
     };
@@ -245,18 +251,24 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     const int b_rd = A_STAGE + fk * LDB_S + wave_n * WAVE_N + frow;
 
     const int ktiles = (k_hi - k_lo + BK - 1) / BK;
+    constexpr std::integral_constant<int, 0> set0{};
+    constexpr std::integral_constant<int, 1> set1{};
     if (ktiles > 0) {
-        load_global(k_lo);
-        store_lds(0);
+        load_global(k_lo, set0);
+        if (ktiles > 1) load_global(k_lo + BK, set1);
+        store_lds(0, set0);
     }
     __syncthreads();
 
-    for (int kt = 0; kt < ktiles; kt++) {
-        const int cur = kt & 1;
-        const bool more = (kt + 1 < ktiles);
-        if (more) load_global(k_lo + (kt + 1) * BK);
+    // Tile kt is multiplied from LDS stage kt % 2.  Its staging set (kt % 2) is free again -- the tile went to
+    // LDS during tile kt - 1 -- and is refilled with tile kt + 2 before the MFMAs; tile kt + 1, requested a
+    // whole tile earlier, goes from the other set to the other LDS stage after them.
+    auto tile = [&](int kt, auto set_c) {
+        constexpr int SET = decltype(set_c)::value;
+        constexpr std::integral_constant<int, SET ^ 1> other{};
+        if (kt + 2 < ktiles) load_global(k_lo + (kt + 2) * BK, set_c);
 
-        const float* sb = smem + cur * STAGE;
+        const float* sb = smem + SET * STAGE;
 #pragma unroll
         for (int s = 0; s < BK / 2; s++) {
             float af[TM], bf[TN];
@@ -271,9 +283,15 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
 
-        if (more) store_lds(cur ^ 1);
+        if (kt + 1 < ktiles) store_lds(SET ^ 1, other);
         __syncthreads();
+    };
+    int kt = 0;
+    for (; kt + 1 < ktiles; kt += 2) {
+        tile(kt, set0);
+        tile(kt + 1, set1);
     }
+    if (kt < ktiles) tile(kt, set0);
 
     // lane l holds column (l % 32); rows 8*(v/4) + 4*(l/32) + (v%4)
     const int col_l = lane & 31, row_l = (lane >> 5) * 4;

@@ -182,10 +182,13 @@ def test_fp32_cost_model_extra_points():
     # one round of 256 tiles: the one-round line; 1024 x 1024 outputs with 64 x 64 tiles
     assert g32.config_cost(key, 30e-6, 1024, 1024, K, pts) == pytest.approx(30e-6)
     assert g32.config_cost(key, 30e-6, 1024, 1024, Ks, pts) == pytest.approx(12e-6)
-    # four rounds at the profile K: later rounds cost the two-round increment (18 us, above half of 30 us)
-    assert g32.config_cost(key, 30e-6, 2048, 2048, K, pts) == pytest.approx(30e-6 + 3 * 18e-6)
-    # at the short K the increment (3 us) is below half a lone round (6 us), so the share applies
-    assert g32.config_cost(key, 30e-6, 2048, 2048, Ks, pts) == pytest.approx(12e-6 + 3 * 6e-6)
+    # four rounds at the profile K: later rounds cost the two-round increment (18 us) or the minimum share of a
+    # lone round (30 us), whichever is larger
+    share = g32.later_round_min_share(K)
+    assert share == g32.LATER_ROUND_MIN_SHARE_SHORT and g32.later_round_min_share(4 * K) == g32.LATER_ROUND_MIN_SHARE_LONG
+    assert g32.config_cost(key, 30e-6, 2048, 2048, K, pts) == pytest.approx(30e-6 + 3 * max(18e-6, share * 30e-6))
+    # at the short K the increment (3 us) is below the share of a lone round (12 us), so the share applies
+    assert g32.config_cost(key, 30e-6, 2048, 2048, Ks, pts) == pytest.approx(12e-6 + 3 * share * 12e-6)
     # a long problem on small tiles is bound by the rate the compute units take operands in
     big = g32.config_cost(key, 20e-6, 8192, 8192, 8192, (12e-6, 30e-6, 15e-6))
     assert big == pytest.approx(4.0 * 8192 ** 3 * (2 / 64) / g32.OPERAND_BYTES_PER_S)
