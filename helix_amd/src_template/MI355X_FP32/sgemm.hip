@@ -60,10 +60,18 @@ typedef int intx4 __attribute__((ext_vector_type(4)));
 
 constexpr int WAVES_M = BM / WAVE_M, WAVES_N = BN / WAVE_N, NWAVES = WAVES_M * WAVES_N, NTHREADS = 64 * NWAVES;
 constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;
-constexpr int LDA_S = BM + 32, LDB_S = BN + 32;              // LDS row strides in floats
-constexpr int A_STAGE = BK * LDA_S, B_STAGE = BK * LDB_S;    // floats
-constexpr int STAGE = A_STAGE + B_STAGE;
-constexpr int LDS_BYTES = 2 * STAGE * 4;
+// LDS row strides in floats.  GEMM mode: +32, which puts the two half-waves of a fragment read on different bank
+// halves and keeps rows 16-byte aligned for the 128-bit tile writes.  CONV mode writes scalars, BK/4 lanes per
+// tile row along k: the extra 16 / (BK/4) floats make the rows those lanes write fall on different banks
+// (4 * stride = 64 / (BK/4) mod 64) instead of all on one.
+constexpr int CONV_PAD = 32 + (BK >= 8 ? 64 / BK : 0);
+template <bool CONV> struct Lds {
+    static constexpr int LDA = BM + (CONV ? CONV_PAD : 32), LDB = BN + (CONV ? CONV_PAD : 32);
+    static constexpr int A_STAGE = BK * LDA, B_STAGE = BK * LDB;    // floats
+    static constexpr int STAGE = A_STAGE + B_STAGE;
+    static constexpr int BYTES = 2 * STAGE * 4;
+};
+constexpr int LDS_BYTES = Lds<true>::BYTES > Lds<false>::BYTES ? Lds<true>::BYTES : Lds<false>::BYTES;
 // GEMM mode: tile rows are k, 16-byte chunks run along m / n
 constexpr int A_CPR = BM / 4, B_CPR = BN / 4;                // chunks per tile row
 constexpr int A_ITERS = BK * A_CPR / NTHREADS, B_ITERS = BK * B_CPR / NTHREADS;
@@ -113,6 +121,7 @@ constexpr int OOB = 0x7fffffff;  // byte offset beyond any buffer: the load retu
 // kernel has its own symbol name and a profiler lists configurations separately.
 template <bool CONV, int T_BM = BM, int T_BN = BN, int T_BK = BK, int T_WM = WAVE_M, int T_WN = WAVE_N>
 __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params p) {
+    constexpr int LDA_S = Lds<CONV>::LDA, LDB_S = Lds<CONV>::LDB, A_STAGE = Lds<CONV>::A_STAGE, STAGE = Lds<CONV>::STAGE;
     extern __shared__ __attribute__((aligned(16))) float smem[];
 
     const int tid = threadIdx.x;
