@@ -754,9 +754,10 @@ inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int
     half_t* col = (half_t*)ws;
     half_t* wp = (half_t*)((unsigned char*)ws + col_bytes);
     void* rest = (unsigned char*)ws + col_bytes + wp_bytes;
-    const helix_im2col::Geom g{H, W, IC, OH, OW, kW, stride, pad, (int)M, (int)K};
+    if (M * (Kp / 8) > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    const helix_im2col::Geom g = helix_im2col::make_geom(H, W, IC, OH, OW, kW, stride, pad, (int)M, (int)K);
     hipLaunchKernelGGL((helix_im2col::im2col_rows_kernel<half_t, 8>), dim3(helix_im2col::grid_for((size_t)M * (Kp / 8))),
-                       dim3(256), 0, s, (const half_t*)x, col, g, Kp);
+                       dim3(256), 0, s, (const half_t*)x, col, g, Kp, helix_fastdiv::make(Kp / 8));
     hipLaunchKernelGGL((helix_im2col::pack_weights_rows_kernel<half_t>), dim3(helix_im2col::grid_for((size_t)OC * Kp)),
                        dim3(256), 0, s, (const half_t*)w, wp, OC, (int)K, Kp);
     hipError_t e = hipGetLastError();

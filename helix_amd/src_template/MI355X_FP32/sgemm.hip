@@ -455,9 +455,10 @@ inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int
     if (!ws || ws_bytes < conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad)) return HELIX_ERR_WORKSPACE;
     float* col = (float*)ws;
     float* wt = (float*)((unsigned char*)ws + col_bytes);
-    const helix_im2col::Geom g{H, W, IC, OH, OW, kW, stride, pad, (int)M, (int)K};
-    hipLaunchKernelGGL((helix_im2col::im2col_cols_kernel<float>), dim3(helix_im2col::grid_for((size_t)K * Mp)), dim3(256),
-                       0, s, (const float*)x, col, g, Mp);
+    const helix_im2col::Geom g = helix_im2col::make_geom(H, W, IC, OH, OW, kW, stride, pad, (int)M, (int)K);
+    hipLaunchKernelGGL((helix_im2col::im2col_cols_kernel<float>),
+                       dim3(helix_im2col::grid_for((size_t)Mp), (unsigned)(K < 65535 ? K : 65535)), dim3(256), 0, s,
+                       (const float*)x, col, g, Mp);
     hipLaunchKernelGGL((helix_im2col::pack_weights_cols_kernel<float>), dim3(helix_im2col::grid_for((size_t)K * Np)),
                        dim3(256), 0, s, (const float*)w, wt, OC, (int)K, Np);
     hipError_t e = hipGetLastError();

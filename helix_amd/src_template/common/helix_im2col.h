@@ -16,54 +16,85 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "helix_fastdiv.h"
+
 namespace helix_im2col {
+
+using helix_fastdiv::FastDiv;
 
 struct Geom {
     int H, W, IC, OH, OW, kW, stride, pad;
     int M, K;   // M = batch*OH*OW, K = kH*kW*IC
+    FastDiv by_OW, by_OH, by_IC, by_kW;   // multiply-shift division by the run-time extents
 };
 
-template <typename T>
-__device__ __forceinline__ T tap(const T* x, const Geom& g, int m, int k) {
-    if (m >= g.M || k >= g.K) return (T)0;
-    const int ow = m % g.OW;
-    const int t = m / g.OW;
-    const int oh = t % g.OH;
-    const int b = t / g.OH;
-    const int c = k % g.IC;
-    const int f = k / g.IC;
-    const int ih = oh * g.stride - g.pad + f / g.kW;
-    const int iw = ow * g.stride - g.pad + f % g.kW;
-    if (ih < 0 || ih >= g.H || iw < 0 || iw >= g.W) return (T)0;
-    return x[(((size_t)b * g.H + ih) * g.W + iw) * g.IC + c];
+inline Geom make_geom(int H, int W, int IC, int OH, int OW, int kW, int stride, int pad, int M, int K) {
+    return Geom{H, W, IC, OH, OW, kW, stride, pad, M, K,
+                helix_fastdiv::make(OW), helix_fastdiv::make(OH), helix_fastdiv::make(IC), helix_fastdiv::make(kW)};
+}
+
+// Output row m -> image base (in pixels) and the image coordinates of its top-left filter tap.
+struct Pixel { int img, ih0, iw0; };
+
+__device__ __forceinline__ Pixel pixel_of(const Geom& g, int m) {
+    const int t = g.by_OW.div(m);
+    const int ow = m - t * g.OW;
+    const int b = g.by_OH.div(t);
+    const int oh = t - b * g.OH;
+    return Pixel{b * g.H * g.W, oh * g.stride - g.pad, ow * g.stride - g.pad};
 }
 
 // K-contiguous column buffer: col[m*ldk + k], k < ldk (ldk a multiple of VEC); one thread writes VEC
-// consecutive k of one row with a single store.
+// consecutive k of one row with a single store.  The row is decomposed once per thread, the first k of the
+// chunk once, and (channel, tap column, tap row) then step from element to element.
+// `by_chunks` divides by ldk / VEC; M * (ldk / VEC) must fit 31 bits (checked by the caller).
 template <typename T, int VEC>
-__global__ void im2col_rows_kernel(const T* x, T* col, Geom g, int ldk) {
-    const int chunks = ldk / VEC;
-    const size_t total = (size_t)g.M * chunks;
-    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (size_t)gridDim.x * blockDim.x) {
-        const int m = (int)(idx / chunks), k0 = (int)(idx % chunks) * VEC;
+__global__ void im2col_rows_kernel(const T* x, T* col, Geom g, int ldk, FastDiv by_chunks) {
+    const int chunks = by_chunks.d;
+    const int total = g.M * chunks;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const int m = by_chunks.div(idx), k0 = (idx - m * chunks) * VEC;
+        const Pixel px = pixel_of(g, m);
+        int f = g.by_IC.div(k0);
+        int c = k0 - f * g.IC;
+        int kh = g.by_kW.div(f);
+        int kw = f - kh * g.kW;
         T v[VEC];
 #pragma unroll
-        for (int j = 0; j < VEC; j++) v[j] = tap(x, g, m, k0 + j);
+        for (int j = 0; j < VEC; j++) {
+            const int ih = px.ih0 + kh, iw = px.iw0 + kw;
+            const bool ok = (k0 + j < g.K) && ih >= 0 && ih < g.H && iw >= 0 && iw < g.W;
+            v[j] = ok ? x[((size_t)px.img + (size_t)ih * g.W + iw) * g.IC + c] : (T)0;
+            if (++c == g.IC) {
+                c = 0;
+                if (++kw == g.kW) { kw = 0; ++kh; }
+            }
+        }
         T* dst = col + (size_t)m * ldk + k0;
 #pragma unroll
         for (int j = 0; j < VEC; j++) dst[j] = v[j];
     }
 }
 
-// M-contiguous column buffer: col[k*ldm + m], m < ldm; consecutive threads write consecutive m.
+// M-contiguous column buffer: col[k*ldm + m], m < ldm.  blockIdx.y walks k (tap and channel are uniform per
+// workgroup), consecutive threads write consecutive m.
 template <typename T>
 __global__ void im2col_cols_kernel(const T* x, T* col, Geom g, int ldm) {
-    const size_t total = (size_t)g.K * ldm;
-    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (size_t)gridDim.x * blockDim.x) {
-        const int k = (int)(idx / ldm), m = (int)(idx % ldm);
-        col[idx] = tap(x, g, m, k);
+    for (int k = blockIdx.y; k < g.K; k += gridDim.y) {
+        const int f = g.by_IC.div(k);
+        const int c = k - f * g.IC;
+        const int kh = g.by_kW.div(f);
+        const int kw = f - kh * g.kW;
+        T* row = col + (size_t)k * ldm;
+        for (int m = blockIdx.x * blockDim.x + threadIdx.x; m < ldm; m += gridDim.x * blockDim.x) {
+            T v = (T)0;
+            if (m < g.M) {
+                const Pixel px = pixel_of(g, m);
+                const int ih = px.ih0 + kh, iw = px.iw0 + kw;
+                if (ih >= 0 && ih < g.H && iw >= 0 && iw < g.W) v = x[((size_t)px.img + (size_t)ih * g.W + iw) * g.IC + c];
+            }
+            row[m] = v;
+        }
     }
 }
 
