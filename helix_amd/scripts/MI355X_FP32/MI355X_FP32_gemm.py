@@ -37,6 +37,7 @@ OPERAND_BYTES_PER_S = 6.5e12
 
 SPLITK_MAX, SPLITK_TARGET, SPLITK_MIN_K = 8, 768, 768   # as in src_template/MI355X_FP32/sgemm.hip
 SPLITK_MIN_K_FEW, SPLITK_FEW_TILES = 256, 128
+SPLITK_MIN_K_TINY, SPLITK_TINY_TILES = 64, 32
 SPLITK_REDUCE_LAUNCH_S = 4e-6   # the reduction kernel of a K-partitioned launch
 
 
@@ -49,7 +50,7 @@ def split_factor(k, M, N, K):
     tiles = math.ceil(M / k[0]) * math.ceil(N / k[1])
     if tiles <= 0 or tiles >= SPLITK_TARGET * 3 // 4:
         return 1
-    min_k = SPLITK_MIN_K_FEW if tiles <= SPLITK_FEW_TILES else SPLITK_MIN_K
+    min_k = SPLITK_MIN_K_TINY if tiles <= SPLITK_TINY_TILES else SPLITK_MIN_K_FEW if tiles <= SPLITK_FEW_TILES else SPLITK_MIN_K
     return max(min(math.ceil(SPLITK_TARGET / tiles), SPLITK_MAX, K // min_k), 1)
 
 

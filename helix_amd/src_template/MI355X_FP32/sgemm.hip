@@ -13,7 +13,8 @@
 // Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N.
 //
 // K partitions: a problem with fewer than 576 output tiles and a long K is split along K over blockIdx.y, up
-// to 8 ways (at least 768 of K each, 256 when there are at most 128 tiles); partial sums go to the caller's workspace
+// to 8 ways (at least 768 of K each, 256 when there are at most 128 tiles, 64 at most 32); partial sums go to the
+// caller's workspace
 // (helix_workspace_bytes) and a second kernel adds them in partition order.  Without the workspace the
 // problem runs unpartitioned.  The reference's FP32 template has no K partition.
 //
@@ -174,10 +175,13 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
         constexpr int SET = decltype(set_c)::value;
         if (!CONV) {
             // rows k0.. of A^T (K x M) starting at column m0; whole rows are inside the buffer, rows >= K are not
-            __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + (size_t)k0 * p.lda + m0,
-                                                  (unsigned)(((size_t)(k_hi - k0) * p.lda - m0) * 4));
-            __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)k0 * p.ldb + n0,
-                                                  (unsigned)(((size_t)(k_hi - k0) * p.ldb - n0) * 4));
+            // past the end of the K range the descriptors are empty: the loads still issue (the wait counts in
+            // front of the LDS writes then never depend on a branch) and return zeros
+            const bool live = k0 < k_hi;
+            __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A + (size_t)(live ? k0 : 0) * p.lda + m0,
+                                                  live ? (unsigned)(((size_t)(k_hi - k0) * p.lda - m0) * 4) : 0u);
+            __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)(live ? k0 : 0) * p.ldb + n0,
+                                                  live ? (unsigned)(((size_t)(k_hi - k0) * p.ldb - n0) * 4) : 0u);
 #pragma unroll
             for (int i = 0; i < NA; i++) {
                 const int c = tid + i * NTHREADS;
@@ -264,7 +268,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     constexpr std::integral_constant<int, 1> set1{};
     if (ktiles > 0) {
         load_global(k_lo, set0);
-        if (ktiles > 1) load_global(k_lo + BK, set1);
+        load_global(k_lo + BK, set1);
         store_lds(0, set0);
     }
     __syncthreads();
@@ -275,7 +279,10 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     auto tile = [&](int kt, auto set_c) {
         constexpr int SET = decltype(set_c)::value;
         constexpr std::integral_constant<int, SET ^ 1> other{};
-        if (kt + 2 < ktiles) load_global(k_lo + (kt + 2) * BK, set_c);
+        load_global(k_lo + (kt + 2) * BK, set_c);       // empty past the end of the K range
+        // the loads stay in front of the MFMAs and of the LDS writes below: sunk behind the writes, their
+        // wait counts would drain the whole queue every tile
+        __builtin_amdgcn_sched_barrier(0);
 
         const float* sb = smem + SET * STAGE;
 #pragma unroll
@@ -292,7 +299,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
         }
 
-        if (kt + 1 < ktiles) store_lds(SET ^ 1, other);
+        __builtin_amdgcn_sched_barrier(0);
+        store_lds(SET ^ 1, other);                       // zeros past the end: the stage is not read again
         __syncthreads();
     };
     int kt = 0;
@@ -361,18 +369,21 @@ inline const char* info_json() {
 // workgroups (three per compute unit: this kernel hides its LDS and global latencies across workgroups that share
 // a compute unit, and a launch of one to two rounds of tiles leaves most units with one), as many as reach
 // the target, at most SPLITK_MAX, and never so many that a partition walks less than SPLITK_MIN_K of K
-// (SPLITK_MIN_K_FEW when the tiles do not even cover half of the compute units).
+// (SPLITK_MIN_K_FEW when the tiles do not even cover half of the compute units, SPLITK_MIN_K_TINY when there are
+// at most 32 of them: a 14 x 14 x 480 -> 192 1x1 convolution went 18 -> 10 us).
 // Measured on 1521 x 768 x 2304: 83 us unpartitioned, 62 us three-way.  The reference's FP32 template has no K
 // partition (src_template/Ampere_FP32/sgemm.cu); its FP16 one is 2-way (gemm_splitK.cu:124-129).
 constexpr int SPLITK_MAX = 8, SPLITK_TARGET = SPLITK_TARGET_BLOCKS, SPLITK_MAX_TILES = SPLITK_TARGET * 3 / 4,
-              SPLITK_MIN_K = 768, SPLITK_MIN_K_FEW = 256, SPLITK_FEW_TILES = 128;
+              SPLITK_MIN_K = 768, SPLITK_MIN_K_FEW = 256, SPLITK_FEW_TILES = 128, SPLITK_MIN_K_TINY = 64,
+              SPLITK_TINY_TILES = 32;
 
 inline int split_factor(long long M, long long N, long long K) {
     const long long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
     if (tiles <= 0 || tiles >= SPLITK_MAX_TILES) return 1;
     long long s = (SPLITK_TARGET + tiles - 1) / tiles;
     if (s > SPLITK_MAX) s = SPLITK_MAX;
-    const long long min_k = tiles <= SPLITK_FEW_TILES ? SPLITK_MIN_K_FEW : SPLITK_MIN_K;
+    const long long min_k = tiles <= SPLITK_TINY_TILES ? SPLITK_MIN_K_TINY
+                            : tiles <= SPLITK_FEW_TILES ? SPLITK_MIN_K_FEW : SPLITK_MIN_K;
     if (s > K / min_k) s = K / min_k;
     return s < 1 ? 1 : (int)s;
 }

@@ -403,7 +403,7 @@ def test_sgemm_f32_k_partitions():
         BM, BN, BK = cfg[:3]
         for (M, N, K) in [(100, 96, 2048), (257, 129, 1000), (64, 64, 8 * BK * 8), (300, 200, 137), (33, 500, 4096)]:
             tiles = -(-M // BM) * -(-N // BN)
-            want_splits = 1 if tiles >= 576 else max(min(-(-768 // tiles), 8, K // (256 if tiles <= 128 else 768)), 1)
+            want_splits = 1 if tiles >= 576 else max(min(-(-768 // tiles), 8, K // (64 if tiles <= 32 else 256 if tiles <= 128 else 768)), 1)
             assert lib.workspace_bytes(M, N, K) == (want_splits * M * N * 4 if want_splits > 1 else 0), (cfg, M, N, K)
             A = seeded_inputs.uniform_pm1((M, K), seeded_inputs.SEED_A)
             B = seeded_inputs.uniform_pm1((K, N), seeded_inputs.SEED_B)
