@@ -4,8 +4,9 @@ Mirrors scripts/Ampere_FP16/Ampere_FP16_conv.py:420-446: the conv is mapped to G
 M = batch*OH*OW, N = OC, K = IC*kH*kW (:432-434), the GEMM cost model picks the configuration, and
 the cost is measured.  The reference runs an im2col executable plus the GEMM executable and adds the
 two times (:437-445); here the selected configuration's library gathers the A tile on the fly (one
-kernel, one time) when IC is a multiple of 8, and runs im2col + weight repack + GEMM on one stream
-inside the same entry point otherwise (one time for the three kernels).
+kernel, one time) when IC is a multiple of 8; otherwise the same entry point first pads the channels of
+activations and weights to a multiple of 8 in its workspace (or, for IC = 1 and 2, runs im2col + weight
+repack + GEMM), all on one stream and timed as one.
 """
 import math
 import os
@@ -22,21 +23,40 @@ root_path = os.getcwd()
 # AlexNet layers, a configuration's conv time exceeds its GEMM prediction by about this fraction per tile
 # column.
 GATHER_COST_PER_TILE_COLUMN = 0.2
+# A K tile that spans several filter taps (IC not a multiple of BLOCK_K: first layers after channel padding,
+# 16- and 24-channel inputs) decomposes the tap per 16-byte chunk instead of once per tile; measured over such
+# layers the time grows by about these fractions per 64 of BLOCK_K and per 128 tile rows.
+GENERAL_GATHER_COST_PER_64_K = 0.3
+GENERAL_GATHER_COST_PER_128_ROWS = 0.2
 
 
-def conv_config_cost(k, v, M, N, K, v_short=None):
-    return config_cost(k, v, M, N, K, v_short) * (1.0 + GATHER_COST_PER_TILE_COLUMN * math.ceil(N / k[2]))
+def conv_config_cost(k, v, M, N, K, v_short=None, IC=None):
+    cost = config_cost(k, v, M, N, K, v_short) * (1.0 + GATHER_COST_PER_TILE_COLUMN * math.ceil(N / k[2]))
+    if IC is not None and IC % k[6]:
+        cost *= (1.0 + GENERAL_GATHER_COST_PER_64_K * k[6] / 64) * (1.0 + GENERAL_GATHER_COST_PER_128_ROWS * k[1] / 128)
+    return cost
 
 
-def cost_model(prof_dict, M, N, K):
+GATHER_CHUNK = 8   # halves per 16-byte chunk of the implicit gather
+
+
+def gather_channels(input_channel):
+    """The channel count the kernel walks: a count off the gather chunk is padded to it in the workspace when
+    that is at most 8/3 of the real one (helix_im2col::pads_channels), otherwise the column-buffer path runs
+    on the real count."""
+    padded = -(-input_channel // GATHER_CHUNK) * GATHER_CHUNK
+    return padded if 3 * padded <= 8 * input_channel else input_channel
+
+
+def cost_model(prof_dict, M, N, K, IC=None):
     """GEMM cost model restricted to the MFMA configurations (the GEMV kernels have no conv path), with the
-    gather term above."""
+    gather terms above; IC is the channel count the kernel walks (gather_channels)."""
     min_cost = float("inf")
     best_config = (1, 1, 1, 1, 1, 0, 32)
     for k, v in prof_dict.items():
         if k[0] == 0:
             continue
-        cost = conv_config_cost(k, v, M, N, K, short_value(prof_dict, k))
+        cost = conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC)
         if min_cost > cost:
             min_cost = cost
             best_config = k
@@ -50,7 +70,7 @@ def get_MI355X_FP16_conv_Helix_result(prof_dict, batch, input_channel, H, W, out
     M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
     N = output_channel
     K = input_channel * kH * kW
-    best_config = cost_model(prof_dict, M, N, K)
+    best_config = cost_model(prof_dict, M, N, gather_channels(input_channel) * kH * kW, gather_channels(input_channel))
     lib = load(library_for_key(best_config))
     _, avg, _ = lib.bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad, warmup=10, iters=10)
     cost = avg * 1e3

@@ -1,7 +1,7 @@
 """Convolution runner of the MI355X_FP32 backend (implicit GEMM, NHWC, FP32).
 Mirrors scripts/Ampere_FP32/Ampere_FP32_conv.py:89-110; one kernel instead of im2col + SGEMM when IC is
-a multiple of 4 (the reference even borrows the FP16 im2col binary here, :107), FP32 im2col + SGEMM
-inside the same entry point otherwise."""
+a multiple of 4 (the reference even borrows the FP16 im2col binary here, :107); otherwise the same entry
+point pads the channels to a multiple of 4 in its workspace first (IC = 1: FP32 im2col + SGEMM)."""
 import math
 import os
 
@@ -23,7 +23,20 @@ def conv_config_cost(k, v, M, N, K, points=None):
     return config_cost(k, v, M, N, K, points) * (1.0 + CONV_COPY_COST_AT_BK32 * k[2] / 32)
 
 
-def cost_model(prof_dict, M, N, K):
+GATHER_CHUNK = 4   # floats per 16-byte chunk of the implicit gather
+
+
+def gather_channels(input_channel):
+    """The channel count the kernel walks: a count off the gather chunk is padded to it in the workspace when
+    that is at most 8/3 of the real one (helix_im2col::pads_channels), otherwise the column-buffer path runs
+    on the real count."""
+    padded = -(-input_channel // GATHER_CHUNK) * GATHER_CHUNK
+    return padded if 3 * padded <= 8 * input_channel else input_channel
+
+
+def cost_model(prof_dict, M, N, K, IC=None):
+    """IC (the channel count the kernel walks) is accepted for symmetry with the FP16 backend; the FP32 gather
+    decomposes the tap per chunk in every case, so no term depends on it."""
     min_cost = float("inf")
     best_config = (1, 1, 1, 1, 1, 1, 1, 1)
     for k, v in prof_dict.items():
@@ -43,7 +56,7 @@ def get_MI355X_FP32_conv_Helix_result(prof_dict, batch, input_channel, H, W, out
     M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
     N = output_channel
     K = input_channel * kH * kW
-    best_config = cost_model(prof_dict, M, N, K)
+    best_config = cost_model(prof_dict, M, N, gather_channels(input_channel) * kH * kW)
     lib = load(library_for_key(best_config))
     _, avg, _ = lib.bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad, warmup=10, iters=10)
     cost = avg * 1e3

@@ -101,7 +101,7 @@ def conv_rows(be, prof_dict, vendor=False):
     for shp in S.get_baseline_conv_shape_list():
         b, ic, h, w, oc, kh, kw, st, pd = shp
         M = b * ((h + 2 * pd - kh) // st + 1) * ((w + 2 * pd - kw) // st + 1)
-        key = be.conv.cost_model(prof_dict, M, oc, ic * kh * kw)
+        key = be.conv.cost_model(prof_dict, M, oc, be.conv.gather_channels(ic) * kh * kw, be.conv.gather_channels(ic))
         ms, tflops = be.conv_result(prof_dict, *shp)
         nbytes = R.conv_bytes(*shp, be.elem_bytes)
         rows.append({"shape": list(shp), "gemm_MNK": [M, oc, ic * kh * kw], "config": list(key), "us": round(ms * 1e3, 2),

@@ -728,8 +728,9 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     return launch<0>(p, ws, ws_bytes, s);
 }
 
-// Convolutions whose channel count is not a multiple of 8 go through a column buffer (K padded to a multiple
-// of 8) and repacked weights in the workspace, then through the GEMM above.
+// Convolutions whose channel count is not a multiple of 8 run on channel-padded copies of activations and
+// weights in the workspace, or (thin inputs, where padding would multiply the work) through a column buffer (K
+// padded to a multiple of 8) and repacked weights there, then through the GEMM above.
 inline int conv_padded_k(int IC, int kH, int kW) { return (IC * kH * kW + 7) / 8 * 8; }
 
 inline size_t conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad) {
@@ -737,9 +738,41 @@ inline size_t conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int 
     const long long M = (long long)batch * OH * OW;
     if (M > 0x7fffffffLL) return 0;
     if (IC % 8 == 0) return workspace_bytes((int)M, OC, IC * kH * kW);
+    if (helix_im2col::pads_channels(batch, H, W, IC, 8, 2)) {
+        const int ICp = helix_im2col::padded_channels(IC, 8);
+        return helix_im2col::align256((size_t)batch * H * W * ICp * 2) +
+               helix_im2col::align256((size_t)OC * kH * kW * ICp * 2) + workspace_bytes((int)M, OC, ICp * kH * kW);
+    }
     const int Kp = conv_padded_k(IC, kH, kW);
     return helix_im2col::align256((size_t)M * Kp * 2) + helix_im2col::align256((size_t)OC * Kp * 2) +
            workspace_bytes((int)M, OC, Kp);
+}
+
+inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
+                  int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s);
+
+inline int conv2d_padded_channels(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC,
+                                  int kH, int kW, int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
+    const int ICp = helix_im2col::padded_channels(IC, 8);
+    const long long pixels = (long long)batch * H * W, taps = (long long)OC * kH * kW;
+    if (taps * (ICp / 8) > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    const size_t xp_bytes = helix_im2col::align256((size_t)pixels * ICp * 2);
+    const size_t wp_bytes = helix_im2col::align256((size_t)taps * ICp * 2);
+    if (!ws || ws_bytes < conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad)) return HELIX_ERR_WORKSPACE;
+    if ((uintptr_t)ws & 15) return HELIX_ERR_INVALID_VALUE;
+    half_t* xp = (half_t*)ws;
+    half_t* wp = (half_t*)((unsigned char*)ws + xp_bytes);
+    const helix_fastdiv::FastDiv by_chunks = helix_fastdiv::make(ICp / 8);
+    hipLaunchKernelGGL((helix_im2col::pad_channels_kernel<half_t, 8>),
+                       dim3(helix_im2col::grid_for((size_t)pixels * (ICp / 8))), dim3(256), 0, s, (const half_t*)x, xp,
+                       (int)pixels, IC, ICp, by_chunks);
+    hipLaunchKernelGGL((helix_im2col::pad_channels_kernel<half_t, 8>),
+                       dim3(helix_im2col::grid_for((size_t)taps * (ICp / 8))), dim3(256), 0, s, (const half_t*)w, wp,
+                       (int)taps, IC, ICp, by_chunks);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return conv2d(xp, wp, y, batch, H, W, ICp, OC, kH, kW, stride, pad, (unsigned char*)ws + xp_bytes + wp_bytes,
+                  ws_bytes - xp_bytes - wp_bytes, s);
 }
 
 inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
@@ -768,8 +801,11 @@ inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int
 inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
                   int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
     if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 1)) return HELIX_ERR_INVALID_VALUE;
-    if (IC % 8 != 0)   // a 16-byte chunk of the implicit gather must stay inside one filter tap
+    if (IC % 8 != 0) {   // a 16-byte chunk of the implicit gather must stay inside one filter tap
+        if (helix_im2col::pads_channels(batch, H, W, IC, 8, 2))
+            return conv2d_padded_channels(x, w, y, batch, H, W, IC, OC, kH, kW, stride, pad, ws, ws_bytes, s);
         return conv2d_explicit(x, w, y, batch, H, W, IC, OC, kH, kW, stride, pad, ws, ws_bytes, s);
+    }
     const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
     const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
     const long long xbytes = (long long)batch * H * W * IC * 2;

@@ -444,16 +444,49 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     return launch<false>(p, ws, ws_bytes, s);
 }
 
-// Convolutions whose channel count is not a multiple of 4 go through a column buffer (K x M, the A layout of
-// this template) and transposed weights (K x N) in the workspace, then through the GEMM above.
+// Convolutions whose channel count is not a multiple of 4 run on channel-padded copies of activations and
+// weights in the workspace, or (IC = 1, where padding would quadruple the work) through a column buffer (K x M,
+// the A layout of this template) and transposed weights (K x N) there, then through the GEMM above.
 inline size_t conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad) {
     const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
     const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
     if (M > 0x7fffffffLL || K > 0x7fffffffLL) return 0;
     if (IC % 4 == 0) return workspace_bytes((int)M, OC, (int)K);
+    if (helix_im2col::pads_channels(batch, H, W, IC, 4, 4)) {
+        const int ICp = helix_im2col::padded_channels(IC, 4);
+        return helix_im2col::align256((size_t)batch * H * W * ICp * 4) +
+               helix_im2col::align256((size_t)OC * kH * kW * ICp * 4) + workspace_bytes((int)M, OC, ICp * kH * kW);
+    }
     const long long Mp = (M + 3) / 4 * 4, Np = (OC + 3) / 4 * 4;
     return helix_im2col::align256((size_t)K * Mp * 4) + helix_im2col::align256((size_t)K * Np * 4) +
            workspace_bytes((int)M, OC, (int)K);
+}
+
+inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
+                  int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s);
+
+inline int conv2d_padded_channels(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC,
+                                  int kH, int kW, int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
+    const int ICp = helix_im2col::padded_channels(IC, 4);
+    const long long pixels = (long long)batch * H * W, taps = (long long)OC * kH * kW;
+    if (taps * (ICp / 4) > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    const size_t xp_bytes = helix_im2col::align256((size_t)pixels * ICp * 4);
+    const size_t wp_bytes = helix_im2col::align256((size_t)taps * ICp * 4);
+    if (!ws || ws_bytes < conv_workspace_bytes(batch, H, W, IC, OC, kH, kW, stride, pad)) return HELIX_ERR_WORKSPACE;
+    if ((uintptr_t)ws & 15) return HELIX_ERR_INVALID_VALUE;
+    float* xp = (float*)ws;
+    float* wp = (float*)((unsigned char*)ws + xp_bytes);
+    const helix_fastdiv::FastDiv by_chunks = helix_fastdiv::make(ICp / 4);
+    hipLaunchKernelGGL((helix_im2col::pad_channels_kernel<float, 4>),
+                       dim3(helix_im2col::grid_for((size_t)pixels * (ICp / 4))), dim3(256), 0, s, (const float*)x, xp,
+                       (int)pixels, IC, ICp, by_chunks);
+    hipLaunchKernelGGL((helix_im2col::pad_channels_kernel<float, 4>),
+                       dim3(helix_im2col::grid_for((size_t)taps * (ICp / 4))), dim3(256), 0, s, (const float*)w, wp,
+                       (int)taps, IC, ICp, by_chunks);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return conv2d(xp, wp, y, batch, H, W, ICp, OC, kH, kW, stride, pad, (unsigned char*)ws + xp_bytes + wp_bytes,
+                  ws_bytes - xp_bytes - wp_bytes, s);
 }
 
 inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
@@ -481,8 +514,11 @@ inline int conv2d_explicit(const void* x, const void* w, void* y, int batch, int
 inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH, int kW,
                   int stride, int pad, void* ws, size_t ws_bytes, hipStream_t s) {
     if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 3)) return HELIX_ERR_INVALID_VALUE;
-    if (IC % 4 != 0)   // a 16-byte chunk of the implicit gather must stay inside one filter tap
+    if (IC % 4 != 0) {   // a 16-byte chunk of the implicit gather must stay inside one filter tap
+        if (helix_im2col::pads_channels(batch, H, W, IC, 4, 4))
+            return conv2d_padded_channels(x, w, y, batch, H, W, IC, OC, kH, kW, stride, pad, ws, ws_bytes, s);
         return conv2d_explicit(x, w, y, batch, H, W, IC, OC, kH, kW, stride, pad, ws, ws_bytes, s);
+    }
     const int OH = (H + 2 * pad - kH) / stride + 1, OW = (W + 2 * pad - kW) / stride + 1;
     const long long M = (long long)batch * OH * OW, K = (long long)kH * kW * IC;
     const long long xbytes = (long long)batch * H * W * IC * 4;

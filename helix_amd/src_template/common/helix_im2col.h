@@ -1,8 +1,14 @@
-// Explicit im2col for the convolution entry points of the MI355X kernel templates: the path taken when the
-// input channel count is not a multiple of the 16-byte chunk the implicit-GEMM gather works in (first layers
-// with IC = 1 or 3, odd channel counts), where the reference's own algorithm -- a column buffer followed by
-// the GEMM (src_template/Ampere_FP16/im2col.cu:38-97, scripts/Ampere_FP16/Ampere_FP16_conv.py:431-446) --
-// is used as is, on NHWC data:
+// The two paths of the convolution entry points for input channel counts that are not a multiple of the
+// 16-byte chunk the implicit-GEMM gather works in (first layers with IC = 1 or 3, odd channel counts).
+//
+// Channel padding (pad_channels_kernel, at the end of this file): activations and weights are copied once with
+// IC rounded up to the chunk, zero-filled, and the implicit gather runs on the copies.  Taken when the
+// padded count is at most 8/3 of IC: the copy moves the input once, where a column buffer is written and
+// read back kH*kW / stride^2 times as large (an 11x11 stride-4 IC = 3 layer at batch 32, FP32: 300 -> 136 us).
+//
+// Explicit im2col, for the thinner inputs (IC = 1, 2 in FP16, 1 in FP32), where padding would multiply
+// the MFMA work by 4 to 8: the reference's own algorithm -- a column buffer followed by the GEMM
+// (src_template/Ampere_FP16/im2col.cu:38-97, scripts/Ampere_FP16/Ampere_FP16_conv.py:431-446) -- on NHWC data:
 //
 //   col[m][k] = x[b][oh*stride - pad + kh][ow*stride - pad + kw][c],   m = (b*OH + oh)*OW + ow,
 //                                                                      k = (kh*kW + kw)*IC + c,
@@ -118,6 +124,33 @@ __global__ void pack_weights_cols_kernel(const T* w, T* out, int N, int K, int l
         const int k = (int)(idx / ldn), n = (int)(idx % ldn);
         out[idx] = n < N ? w[(size_t)n * K + k] : (T)0;
     }
+}
+
+// rows x IC -> rows x ICp (ICp a multiple of VEC, >= IC), zero-filled tail; serves NHWC activations (one row
+// per pixel) and [OC][kH][kW][IC] weights (one row per filter tap) alike.  One thread writes VEC consecutive
+// channels of one row with a single store.  `by_chunks` divides by ICp / VEC; rows * (ICp / VEC) must fit 31 bits.
+template <typename T, int VEC>
+__global__ void pad_channels_kernel(const T* src, T* dst, int rows, int IC, int ICp, FastDiv by_chunks) {
+    const int chunks = by_chunks.d;
+    const int total = rows * chunks;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        const int r = by_chunks.div(idx), c0 = (idx - r * chunks) * VEC;
+        const T* from = src + (size_t)r * IC + c0;
+        struct alignas(sizeof(T) * VEC) Chunk { T v[VEC]; } chunk;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) chunk.v[j] = (c0 + j < IC) ? from[j] : (T)0;
+        *reinterpret_cast<Chunk*>(dst + (size_t)r * ICp + c0) = chunk;   // dst is aligned to the chunk by the caller
+    }
+}
+
+// Channel count after padding to the gather chunk of VEC elements, and whether that path is the one taken:
+// the padded count within 8/3 of IC and the padded activations within the 2 GiB a buffer descriptor spans.
+inline int padded_channels(int IC, int vec) { return (IC + vec - 1) / vec * vec; }
+
+inline bool pads_channels(int batch, int H, int W, int IC, int vec, int elem_bytes) {
+    const int ICp = padded_channels(IC, vec);
+    return IC % vec != 0 && 3LL * ICp <= 8LL * IC &&
+           (long long)batch * H * W * ICp * elem_bytes < 0x7fffffffLL;
 }
 
 inline int grid_for(size_t total) {

@@ -66,14 +66,16 @@ int helix_gemm(const void* A, const void* B, void* C, int M, int N, int K, int l
                void* workspace, size_t workspace_bytes, void* stream);
 
 /* Bytes of device scratch `helix_conv2d` needs for this problem: the split-K partial sums of the implicit
- * GEMM, or -- when IC is not a multiple of the 16-byte gather chunk (8 halves / 4 floats) -- the column
- * buffer and repacked weights of the explicit im2col path plus what its GEMM needs.
+ * GEMM, plus -- when IC is not a multiple of the 16-byte gather chunk (8 halves / 4 floats) -- the
+ * channel-padded copies of activations and weights, or (IC = 1; 2 in FP16) the column buffer and repacked
+ * weights of the explicit im2col path.
  * Replaces: the `col` buffer the reference's im2col executable allocates for itself
  * (src_template/Ampere_FP16/im2col.cu:140-150). */
 size_t helix_conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad);
 
 /* One NHWC convolution on `stream`: implicit GEMM (no column buffer) when IC is a multiple of the gather
- * chunk, else im2col into the workspace followed by the GEMM, as the reference does for every layer.
+ * chunk; else the same on copies with the channels zero-padded to the chunk, or (IC = 1; 2 in FP16) im2col
+ * into the workspace followed by the GEMM, as the reference does for every layer.
  * Replaces: `im2col batch IC H W OC kH kW stride pad` followed by the GEMM executable
  * (scripts/Ampere_FP16/Ampere_FP16_conv.py:431-446, src_template/Ampere_FP16/im2col.cu:38-97). */
 int helix_conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,

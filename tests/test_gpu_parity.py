@@ -275,9 +275,10 @@ def run_conv(lib, x, w, stride, pad, dtype):
 CONV_GEOMS = [(2, 14, 14, 16, 24, 3, 3, 1, 1), (2, 15, 13, 8, 8, 3, 3, 2, 1), (3, 8, 8, 32, 16, 1, 1, 2, 0),
               (1, 12, 12, 8, 40, 5, 5, 1, 2), (2, 9, 9, 64, 64, 3, 3, 1, 1), (1, 7, 7, 24, 16, 3, 3, 1, 0),
               (2, 6, 10, 72, 8, 1, 1, 1, 0)]
-# channel counts that are not a multiple of the gather chunk: explicit im2col + GEMM through the workspace
+# channel counts that are not a multiple of the gather chunk: channel-padded copies in the workspace (IC = 3, 6,
+# 25; 2 in FP32) or explicit im2col + GEMM through the workspace (IC = 1; 2 in FP16)
 CONV_GEOMS_ODD = [(2, 20, 20, 3, 16, 7, 7, 2, 3), (1, 9, 11, 1, 8, 5, 5, 2, 0), (2, 8, 8, 25, 24, 5, 5, 1, 2),
-                  (1, 10, 10, 6, 10, 3, 3, 1, 1), (3, 13, 13, 3, 96, 11, 11, 4, 0)]
+                  (1, 10, 10, 6, 10, 3, 3, 1, 1), (3, 13, 13, 3, 96, 11, 11, 4, 0), (2, 7, 9, 2, 8, 3, 3, 1, 1)]
 
 
 @pytest.mark.parametrize("cfg", [(2, 128, 128, 64, 64, 64), (2, 64, 64, 32, 32, 64), (2, 256, 64, 64, 32, 64),
@@ -311,19 +312,28 @@ def test_conv_f16_golden_and_special_cases():
     wi = rng.integers(-2, 3, (16, 3, 3, 8)).astype(np.float16)
     want = O.conv2d_nhwc(xi.astype(np.float32), wi.astype(np.float32), 2, 1)
     assert np.array_equal(run_conv(lib, xi, wi, 2, 1, torch.float16).astype(np.float32), want)
-    # IC = 3 takes the column-buffer path: exact on integers too, also through a split-K library, and refused
-    # without its workspace rather than mis-computed
+    # IC = 3 runs on channel-padded copies, IC = 1 through the column buffer: exact on integers too, also through a
+    # split-K library, and refused without the workspace rather than mis-computed
     xi3 = rng.integers(-2, 3, (2, 9, 8, 3)).astype(np.float16)
     wi3 = rng.integers(-2, 3, (16, 3, 3, 3)).astype(np.float16)
     want3 = O.conv2d_nhwc(xi3.astype(np.float32), wi3.astype(np.float32), 2, 1)
     assert np.array_equal(run_conv(lib, xi3, wi3, 2, 1, torch.float16).astype(np.float32), want3)
     libk = load(b16.kernel_library("gemm_splitK", 2, 64, 64, 32, 32, 64))
     assert np.array_equal(run_conv(libk, xi3, wi3, 2, 1, torch.float16).astype(np.float32), want3)
-    assert lib.conv_workspace_bytes(1, 8, 8, 3, 8, 3, 3, 1, 1) >= 64 * 32 * 2 + 8 * 32 * 2
+    xi1 = rng.integers(-2, 3, (2, 9, 8, 1)).astype(np.float16)
+    wi1 = rng.integers(-2, 3, (16, 3, 3, 1)).astype(np.float16)
+    want1 = O.conv2d_nhwc(xi1.astype(np.float32), wi1.astype(np.float32), 2, 1)
+    for l in (lib, libk):
+        assert np.array_equal(run_conv(l, xi1, wi1, 2, 1, torch.float16).astype(np.float32), want1)
+    # padded copies: 64 pixels and 72 filter taps of 8 halves, each rounded up to 256 bytes
+    assert lib.conv_workspace_bytes(1, 8, 8, 3, 8, 3, 3, 1, 1) == 64 * 8 * 2 + 1280
+    # column buffer: 64 rows and 8 filters of K = 9 padded to 16 halves
+    assert lib.conv_workspace_bytes(1, 8, 8, 1, 8, 3, 3, 1, 1) >= 64 * 16 * 2 + 8 * 16 * 2
     assert lib.conv_workspace_bytes(1, 8, 8, 8, 8, 3, 3, 1, 1) == 0
     t = torch.zeros(4096, dtype=torch.float16, device="cuda:0")
-    assert lib.conv2d(t.data_ptr(), t.data_ptr(), t.data_ptr(), 1, 8, 8, 3, 8, 3, 3, 1, 1, check=False) == \
-        HELIX_ERR_WORKSPACE
+    for ic in (3, 1):
+        assert lib.conv2d(t.data_ptr(), t.data_ptr(), t.data_ptr(), 1, 8, 8, ic, 8, 3, 3, 1, 1, check=False) == \
+            HELIX_ERR_WORKSPACE
 
 
 def test_conv_f16_baseline_layers_sampled():

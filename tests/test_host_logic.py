@@ -20,6 +20,7 @@ from MI355X_FP16 import benchmark_MI355X_FP16_performance_comparison as cmp16
 from MI355X_FP32 import build_MI355X_FP32 as b32
 from MI355X_FP32 import profile_MI355X_FP32 as p32
 from MI355X_FP32 import MI355X_FP32_gemm as g32
+from MI355X_FP32 import MI355X_FP32_conv as c32
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 N_FP16_CONFIGS = 159   # points of the FP16 template space (tile x wave tile x BLOCK_K) that fit LDS and registers
@@ -164,6 +165,14 @@ def test_fp16_cost_model_two_point_profile():
     # conv: every column of tiles gathers its rows again
     assert c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6) == \
         pytest.approx(g16.config_cost(big, 60e-6, 4096, 512, K, 8e-6) * (1 + 2 * c16.GATHER_COST_PER_TILE_COLUMN))
+    # a K tile spanning several filter taps (IC not a multiple of BLOCK_K) pays the per-chunk tap decomposition
+    assert c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6, IC=big[6]) == c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6)
+    assert c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6, IC=8) == pytest.approx(
+        c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6) * (1 + c16.GENERAL_GATHER_COST_PER_64_K * big[6] / 64)
+        * (1 + c16.GENERAL_GATHER_COST_PER_128_ROWS * big[1] / 128))
+    # channel counts off the gather chunk: padded when that is at most 8/3 of the real count, else left alone
+    assert [c16.gather_channels(c) for c in (1, 2, 3, 6, 8, 25, 64)] == [1, 2, 8, 8, 8, 32, 64]
+    assert [c32.gather_channels(c) for c in (1, 2, 3, 6, 8, 25, 64)] == [1, 4, 4, 8, 8, 28, 64]
     # GEMV rows: 9 or more activation rows run the K-partitioned MFMA variant (higher floor); the split-K
     # GEMV library pays its reduction
     assert g16.config_cost((0, 16, 128, 0, 0, 0, 0), 1e-9, 13, 128, 512) == g16.GEMV_MFMA_FLOOR_S
