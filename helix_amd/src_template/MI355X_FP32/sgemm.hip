@@ -171,6 +171,38 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
         }
     }
 
+    // CONV: buffer descriptors of the whole input and of this tile's weight rows (N x K row-major; rows >= N fall
+    // outside), and the byte offsets of the next K tile to request: conv_offsets(k0) fills them for the tile at k0
+    // (index arithmetic only), load_global then issues the loads from them.
+    const int rows_b = (p.N - n0) < BN ? (p.N - n0) : BN;
+    const __amdgpu_buffer_rsrc_t conv_ra = make_rsrc(p.A, CONV ? p.a_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t conv_rb =
+        make_rsrc(p.B + (CONV ? (size_t)n0 * p.K : 0), CONV ? (unsigned)((size_t)rows_b * p.K * 4) : 0u);
+    int off_a[NA], off_b[NB];
+    auto conv_offsets = [&](int k0) {
+        const int k = k0 + (tid % K_CPR) * 4;
+        const bool dead = k >= k_hi;
+        const int t = p.g.by_IC.div(k);
+        const int c = k - t * p.g.IC;
+        const int kh = p.g.by_kW.div(t);
+        const int kw = t - kh * p.g.kW;
+#pragma unroll
+        for (int i = 0; i < NA; i++) {
+            const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
+            // no short-circuit evaluation and the offset computed either way: branches or predicated blocks here
+            // would cut the tile's MFMA block into pieces
+            const bool ok = (!dead) & (cv_img[i] >= 0) & ((unsigned)ih < (unsigned)p.g.H) & ((unsigned)iw < (unsigned)p.g.W);
+            const int off = ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 4;
+            off_a[i] = ok ? off : OOB;
+        }
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const int n = (tid + i * NTHREADS) / K_CPR;
+            const int off = (n * p.K + k) * 4;
+            off_b[i] = dead ? OOB : off;
+        }
+    };
+
     auto load_global = [&](int k0, auto set_c) {
         constexpr int SET = decltype(set_c)::value;
         if (!CONV) {
@@ -193,28 +225,11 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
                 stage_b[SET][i] = buf_load16(rb, ((c / B_CPR) * p.ldb + (c % B_CPR) * 4) * 4);
             }
         } else {
-            __amdgpu_buffer_rsrc_t ra = make_rsrc(p.A, p.a_bytes);
-            const int kc = tid % K_CPR;
-            const int k = k0 + kc * 4;
-            const bool dead = k >= k_hi;
-            const int t = p.g.by_IC.div(k);
-            const int c = k - t * p.g.IC;
-            const int kh = p.g.by_kW.div(t);
-            const int kw = t - kh * p.g.kW;
+            // the offsets were computed a tile earlier (conv_offsets), among that tile's MFMAs
 #pragma unroll
-            for (int i = 0; i < NA; i++) {
-                const int ih = cv_ih[i] + kh, iw = cv_iw[i] + kw;
-                const bool ok = !dead && cv_img[i] >= 0 && ih >= 0 && ih < p.g.H && iw >= 0 && iw < p.g.W;
-                stage_a[SET][i] = buf_load16(ra, ok ? ((cv_img[i] + ih * p.g.W + iw) * p.g.IC + c) * 4 : OOB);
-            }
-            // weights: N x K row-major; rows >= N fall outside the buffer
-            const int rows_b = (p.N - n0) < BN ? (p.N - n0) : BN;
-            __amdgpu_buffer_rsrc_t rb = make_rsrc(p.B + (size_t)n0 * p.K, (unsigned)((size_t)rows_b * p.K * 4));
+            for (int i = 0; i < NA; i++) stage_a[SET][i] = buf_load16(conv_ra, off_a[i]);
 #pragma unroll
-            for (int i = 0; i < NB; i++) {
-                const int n = (tid + i * NTHREADS) / K_CPR;
-                stage_b[SET][i] = buf_load16(rb, dead ? OOB : (n * p.K + k) * 4);
-            }
+            for (int i = 0; i < NB; i++) stage_b[SET][i] = buf_load16(conv_rb, off_b[i]);
         }
     };
 
@@ -267,8 +282,11 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     constexpr std::integral_constant<int, 0> set0{};
     constexpr std::integral_constant<int, 1> set1{};
     if (ktiles > 0) {
+        if (CONV) conv_offsets(k_lo);
         load_global(k_lo, set0);
+        if (CONV) conv_offsets(k_lo + BK);
         load_global(k_lo + BK, set1);
+        if (CONV) conv_offsets(k_lo + 2 * BK);
         store_lds(0, set0);
     }
     __syncthreads();
@@ -283,6 +301,13 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
         // the loads stay in front of the MFMAs and of the LDS writes below: sunk behind the writes, their
         // wait counts would drain the whole queue every tile
         __builtin_amdgcn_sched_barrier(0);
+        // CONV: the gather offsets of tile kt + 3, free to be scheduled among the MFMAs below (computed in front
+        // of their own loads they ran while the matrix pipe sat idle: all waves leave the barrier together)
+        if (CONV) {
+            int k_next = k_lo + (kt + 3) * BK;
+            asm volatile("" : "+s"(k_next));   // keeps the arithmetic that follows on this side of the fence above
+            conv_offsets(k_next);
+        }
 
         const float* sb = smem + SET * STAGE;
 #pragma unroll
@@ -297,6 +322,16 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 #pragma unroll
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+        if (CONV) {
+            // issue order of the block above: the index arithmetic of conv_offsets dealt out behind the MFMAs, a
+            // few instructions each (fragment reads are left to the scheduler, which keeps them a k step ahead)
+            constexpr int MFMA = 0x008, VALU = 0x002, VALU_PER_MFMA = 3;
+#pragma unroll
+            for (int q = 0; q < (BK / 2) * TM * TN; q++) {
+                __builtin_amdgcn_sched_group_barrier(MFMA, 1, SET);
+                __builtin_amdgcn_sched_group_barrier(VALU, VALU_PER_MFMA, SET);
+            }
         }
 
         __builtin_amdgcn_sched_barrier(0);
