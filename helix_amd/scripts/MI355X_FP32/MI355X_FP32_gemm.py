@@ -18,17 +18,14 @@ GEMV_LAUNCH_FLOOR_S = 3.4e-6
 # for them no longer holds (measured: 661 x 768 x 3072 FP32, 103 us against 27 us)
 GEMV_MAX_ROWS = 16
 GEMV_SPLITK_EXTRA_S = 2e-6        # the K-partitioned library's reduction pass on a problem too small to need it
-# a further round of tiles costs what the two-round profile shows beyond one round, but never less than a share of
-# a lone round: the profiled problems sit in the caches, long ones do not.  The share grows with the K a workgroup
-# walks (workgroups sharing a compute unit overlap each other's latencies on short walks; on long ones they compete
-# for the caches): SHORT up to the profile K, LONG from four times that, linear in between.
-LATER_ROUND_MIN_SHARE_SHORT = 0.5
-LATER_ROUND_MIN_SHARE_LONG = 0.85
-
-
-def later_round_min_share(k_walk):
-    t = min(max((k_walk - PROFILE_K) / (3.0 * PROFILE_K), 0.0), 1.0)
-    return LATER_ROUND_MIN_SHARE_SHORT + (LATER_ROUND_MIN_SHARE_LONG - LATER_ROUND_MIN_SHARE_SHORT) * t
+# a further round of tiles costs what the two-round profile shows beyond one round, but never less than the matrix
+# pipes need for it at this fraction of their peak: the small-tile configurations fit several workgroups on a
+# compute unit, so their second round is almost free in the profile and stays so only until the pipes are full
+FP32_MFMA_FLOPS = 157.3e12
+LATER_ROUND_MFMA_FRACTION = 0.85
+# configurations with BK = 32 (one wave group) measure about this much slower over several rounds than their
+# one- and two-round profile points predict (140 GEMM shapes, every configuration timed on each)
+BK32_MULTI_ROUND_COST = 0.05
 
 # rate at which the compute units take A and B tiles in (bytes of M*N*K*4*(1/BM + 1/BN) per second): what the
 # small-tile configurations reach on 2048^3 ... 8192^3
@@ -66,7 +63,7 @@ def config_cost(k, v, M, N, K, points=None):
     """rounds * time-per-round as in Ampere_FP32_gemm.py:93-95, with 256 compute units for 108 SMs and
     the round time following K (the reference ignores K).  `points` = (short, two_rounds, short_two_rounds)
     of the profile when it holds them: then the first round costs the line through the two one-round points
-    and each further round the line through the two-round increments."""
+    and each further round the line through the two-round increments, floored by the matrix pipes' time for it."""
     if k[2] == 0:
         small, big = (M, N) if M <= N else (N, M)
         if small > GEMV_MAX_ROWS:
@@ -88,9 +85,13 @@ def config_cost(k, v, M, N, K, points=None):
     short, two, short_two = points
     first = max(_line(PROFILE_K_SHORT, short, PROFILE_K, v, k_walk), 0.25 * short)
     later = _line(PROFILE_K_SHORT, short_two - short, PROFILE_K, two - v, k_walk)
-    later = min(max(later, later_round_min_share(k_walk) * first), first)
+    mfma_round = 2.0 * NUM_CU * k[0] * k[1] * k_walk / (LATER_ROUND_MFMA_FRACTION * FP32_MFMA_FLOPS)
+    later = min(max(later, mfma_round), first)
     operand_floor = 4.0 * tiles_m * k[0] * tiles_n * k[1] * K * (1 / k[0] + 1 / k[1]) / OPERAND_BYTES_PER_S
-    return max(first + (w - 1) * later + reduce, hbm_floor, operand_floor)
+    cost = max(first + (w - 1) * later + reduce, hbm_floor, operand_floor)
+    if k[2] == 32 and k[6] == 1 and w >= 2:
+        cost *= 1.0 + BK32_MULTI_ROUND_COST
+    return cost
 
 
 def extra_points(prof_dict, k):

@@ -20,16 +20,27 @@ WAVE_TILE_LIST = [32, 64, 128]
 BLOCK_SCALE_LIST = [1, 2, 4]
 BK_LIST = [8, 16, 32]
 LDS_LIMIT = 160 * 1024
+# K-group configurations: several waves per 32 x 32 wave tile, each multiplying a slice of every K tile.  An
+# accumulator is a chain of K / 2 dependent MFMAs whatever the tile shape, so problems of few tiles and long K
+# (transformer projections of a few hundred tokens, the last layers of a CNN) finish sooner with the chain cut
+# inside the workgroup; deep K tiles keep enough bytes in flight for the few workgroups there are.
+KGROUP_BLOCK_SCALES = [(1, 1), (1, 2), (2, 1), (2, 2)]
+KGROUP_BK_KG_LIST = [(32, 2), (32, 4), (64, 2), (64, 4), (128, 8)]
 
 
-def is_valid_config(BMt, BNt, BM, BN, BK=16, WAVE_M=64, WAVE_N=64):
+def is_valid_config(BMt, BNt, BM, BN, BK=16, WAVE_M=64, WAVE_N=64, KG=1):
     # reference rules (build_Ampere_FP32.py:7-12): fewer than 512 threads' worth of tiles, tile extent bounds
-    if BMt * BNt * 64 > 512:
+    # (a full 1024-thread workgroup when the waves also divide K among themselves)
+    if BMt * BNt * 64 * KG > (512 if KG == 1 else 1024):
         return False
     if BM > 256 or BN > 256 or BM < 32 or BN < 32:
         return False
     # gfx950 resources
-    threads = 64 * BMt * BNt
+    threads = 64 * BMt * BNt * KG
+    if (BK // 2) % KG:                                             # whole MFMA k steps per wave group
+        return False
+    if (KG - 1) * BM * BN * 4 > LDS_LIMIT:                         # partial tiles of the groups, added through LDS
+        return False
     if (BK * BM // 4) % threads or (BK * BN // 4) % threads:       # GEMM tile copy, 16-byte chunks along M / N
         return False
     if (BM * BK // 4) % threads or (BN * BK // 4) % threads:       # conv tile copy, 16-byte chunks along K
@@ -56,8 +67,19 @@ def iter_configs():
                         yield (BM, BN, BK, WAVE_M, WAVE_N)
 
 
-def sgemm_library(BM, BN, BK, WAVE_M, WAVE_N):
-    return f"{bin_dir('fp32')}/libsgemm_{BM}_{BN}_{BK}_{WAVE_M}_{WAVE_N}.so"
+def iter_kgroup_configs():
+    """Yields (BM, BN, BK, WAVE_M, WAVE_N, K_GROUPS) of the K-group configurations in build order."""
+    WAVE_M = WAVE_N = 32
+    for (BK, KG) in KGROUP_BK_KG_LIST:
+        for (BMt, BNt) in KGROUP_BLOCK_SCALES:
+            BM, BN = BMt * WAVE_M, BNt * WAVE_N
+            if is_valid_config(BMt, BNt, BM, BN, BK, WAVE_M, WAVE_N, KG):
+                yield (BM, BN, BK, WAVE_M, WAVE_N, KG)
+
+
+def sgemm_library(BM, BN, BK, WAVE_M, WAVE_N, KG=1):
+    suffix = "" if KG == 1 else f"_kg{KG}"
+    return f"{bin_dir('fp32')}/libsgemm_{BM}_{BN}_{BK}_{WAVE_M}_{WAVE_N}{suffix}.so"
 
 
 def kernel_library(kernel_name):
@@ -70,17 +92,23 @@ def default_library():
 
 
 def library_for_key(key):
-    """prof-dict key -> library.  key = (BM, BN, BK, WAVE_M, WAVE_N, LDS_STAGES, COPY_A, COPY_B) keeps the
+    """prof-dict key -> library.  key = (BM, BN, BK, WAVE_M, WAVE_N, LDS_STAGES, K_GROUPS, COPY_VEC) keeps the
     reference's eight fields with BM, BN, BK in the same places (profile_Ampere_FP32.py:46); BK == 0 marks
     the GEMV rows, whose first two fields are the activation-row tile and 128 weight rows."""
     if key[2] == 0:
         return kernel_library("gemv_fp32" if key[5] == 0 else "gemv_fp32_splitK")
-    return sgemm_library(key[0], key[1], key[2], key[3], key[4])
+    return sgemm_library(key[0], key[1], key[2], key[3], key[4], key[6])
 
 
-def compile_sgemm(BM, BN, BK, WAVE_M, WAVE_N):
+def config_key(BM, BN, BK, WAVE_M, WAVE_N, KG=1):
+    return (BM, BN, BK, WAVE_M, WAVE_N, 2, KG, 4)
+
+
+def compile_sgemm(BM, BN, BK, WAVE_M, WAVE_N, KG=1):
     defines = {"BM": BM, "BN": BN, "BK": BK, "WAVE_M": WAVE_M, "WAVE_N": WAVE_N}
-    return (f"{SRC_ROOT}/MI355X_FP32/sgemm.hip", sgemm_library(BM, BN, BK, WAVE_M, WAVE_N), defines)
+    if KG != 1:
+        defines["K_GROUPS"] = KG
+    return (f"{SRC_ROOT}/MI355X_FP32/sgemm.hip", sgemm_library(BM, BN, BK, WAVE_M, WAVE_N, KG), defines)
 
 
 def compile_kernel(kernel_name):
@@ -94,6 +122,7 @@ def compile_kernel(kernel_name):
 
 def build_jobs():
     jobs = [compile_sgemm(*cfg) for cfg in iter_configs()]
+    jobs += [compile_sgemm(*cfg) for cfg in iter_kgroup_configs()]
     jobs.append(compile_kernel("gemv_fp32"))
     jobs.append(compile_kernel("gemv_fp32_splitK"))
     jobs.append(rocblas_job())

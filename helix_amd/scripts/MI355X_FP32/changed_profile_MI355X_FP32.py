@@ -4,7 +4,8 @@ import os
 from tqdm import tqdm
 
 from utils.helix_runtime import write_prof_dict
-from MI355X_FP32.build_MI355X_FP32 import WAVE_TILE_LIST, BLOCK_SCALE_LIST, BK_LIST, is_valid_config
+from MI355X_FP32.build_MI355X_FP32 import WAVE_TILE_LIST, BLOCK_SCALE_LIST, BK_LIST, is_valid_config, config_key, \
+    iter_kgroup_configs
 from MI355X_FP32.profile_MI355X_FP32 import time_config, GEMV_KEYS, GEMV_SPLITK_KEYS
 
 root_path = os.getcwd()
@@ -23,14 +24,15 @@ def profile_Helix_MI355X_FP32_gemm_kernel():
                     pbar.update(1)
                     if not is_valid_config(1, 1, WAVE_M, WAVE_N, BK, WAVE_M, WAVE_N):
                         continue
-                    cost = time_config((WAVE_M, WAVE_N, BK, WAVE_M, WAVE_N, 2, 4, 4))
+                    cost = time_config(config_key(WAVE_M, WAVE_N, BK, WAVE_M, WAVE_N))
                     for BMt in BLOCK_SCALE_LIST:
                         for BNt in BLOCK_SCALE_LIST:
                             BM, BN = BMt * WAVE_M, BNt * WAVE_N
                             if not is_valid_config(BMt, BNt, BM, BN, BK, WAVE_M, WAVE_N):
                                 continue
-                            prof_dict[(BM, BN, BK, WAVE_M, WAVE_N, 2, 4, 4)] = float(cost) * BMt * BNt
-        for key in GEMV_KEYS + GEMV_SPLITK_KEYS:
+                            prof_dict[config_key(BM, BN, BK, WAVE_M, WAVE_N)] = float(cost) * BMt * BNt
+        # the few K-group configurations and the GEMV rows are timed one by one
+        for key in [config_key(*cfg) for cfg in iter_kgroup_configs()] + GEMV_KEYS + GEMV_SPLITK_KEYS:
             prof_dict[key] = time_config(key)
         pbar.update(1)
 

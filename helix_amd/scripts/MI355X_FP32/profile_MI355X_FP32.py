@@ -9,7 +9,7 @@ from tqdm import tqdm
 
 from utils.helix_runtime import load, write_prof_dict, ProfDict
 from utils.roofline import NUM_CU
-from MI355X_FP32.build_MI355X_FP32 import iter_configs, library_for_key
+from MI355X_FP32.build_MI355X_FP32 import iter_configs, iter_kgroup_configs, config_key, library_for_key
 
 root_path = os.getcwd()
 
@@ -44,7 +44,7 @@ def time_config(key, warmup=3, iters=10, K=PROFILE_K, rounds=PROFILE_ROUNDS, per
 
 
 def all_keys():
-    keys = [(BM, BN, BK, WAVE_M, WAVE_N, 2, 4, 4) for (BM, BN, BK, WAVE_M, WAVE_N) in iter_configs()]
+    keys = [config_key(*cfg) for cfg in iter_configs()] + [config_key(*cfg) for cfg in iter_kgroup_configs()]
     return keys + GEMV_KEYS + GEMV_SPLITK_KEYS
 
 

@@ -46,6 +46,9 @@
 #ifndef WAVE_N
 #define WAVE_N 64
 #endif
+#ifndef K_GROUPS
+#define K_GROUPS 1   // groups of waves that share one output tile and each take a slice of every K tile
+#endif
 #ifndef GROUP_ROWS
 #define GROUP_ROWS 8
 #endif
@@ -59,8 +62,16 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef int intx4 __attribute__((ext_vector_type(4)));
 
-constexpr int WAVES_M = BM / WAVE_M, WAVES_N = BN / WAVE_N, NWAVES = WAVES_M * WAVES_N, NTHREADS = 64 * NWAVES;
+// K_GROUPS > 1: the workgroup holds K_GROUPS waves per wave tile.  An accumulator is a chain of dependent MFMAs,
+// K / 2 of them at 64 cycles each, whatever the tile shape: a problem of few tiles and long K is bound by that
+// chain (and by the few bytes its workgroups keep in flight), so the waves of a group each multiply BK / K_GROUPS
+// of every K tile and the partial tiles are added through LDS at the end -- the K partitioning of a split-K
+// launch, inside the workgroup and without the second kernel.
+constexpr int KG = K_GROUPS;
+constexpr int WAVES_M = BM / WAVE_M, WAVES_N = BN / WAVE_N, WAVES_MN = WAVES_M * WAVES_N, NWAVES = WAVES_MN * KG,
+              NTHREADS = 64 * NWAVES;
 constexpr int TM = WAVE_M / 32, TN = WAVE_N / 32;
+constexpr int KSTEPS = BK / 2 / KG;   // MFMA k steps (2 of K each) of one wave per K tile
 // LDS row strides in floats.  GEMM mode: +32, which puts the two half-waves of a fragment read on different bank
 // halves and keeps rows 16-byte aligned for the 128-bit tile writes.  CONV mode writes scalars, BK/4 lanes per
 // tile row along k: the extra 16 / (BK/4) floats make the rows those lanes write fall on different banks
@@ -72,7 +83,9 @@ template <bool CONV> struct Lds {
     static constexpr int STAGE = A_STAGE + B_STAGE;
     static constexpr int BYTES = 2 * STAGE * 4;
 };
-constexpr int LDS_BYTES = Lds<true>::BYTES > Lds<false>::BYTES ? Lds<true>::BYTES : Lds<false>::BYTES;
+constexpr int REDUCE_BYTES = (KG - 1) * BM * BN * 4;   // partial tiles of the wave groups beyond the first
+constexpr int STAGES_BYTES = Lds<true>::BYTES > Lds<false>::BYTES ? Lds<true>::BYTES : Lds<false>::BYTES;
+constexpr int LDS_BYTES = STAGES_BYTES > REDUCE_BYTES ? STAGES_BYTES : REDUCE_BYTES;
 // GEMM mode: tile rows are k, 16-byte chunks run along m / n
 constexpr int A_CPR = BM / 4, B_CPR = BN / 4;                // chunks per tile row
 constexpr int A_ITERS = BK * A_CPR / NTHREADS, B_ITERS = BK * B_CPR / NTHREADS;
@@ -83,6 +96,7 @@ constexpr int AC_ITERS = BM * K_CPR / NTHREADS, BC_ITERS = BN * K_CPR / NTHREADS
 static_assert(BM % WAVE_M == 0 && BN % WAVE_N == 0, "block tile must be a multiple of the wave tile");
 static_assert(WAVE_M % 32 == 0 && WAVE_N % 32 == 0, "wave tile is built from 32x32 MFMA tiles");
 static_assert(BK % 4 == 0 && BK >= 4, "BK must be a multiple of 4");
+static_assert(KG >= 1 && (BK / 2) % KG == 0, "the k steps of a K tile must divide among the wave groups");
 static_assert(NTHREADS <= 1024, "too many waves");
 static_assert((BK * A_CPR) % NTHREADS == 0 && (BK * B_CPR) % NTHREADS == 0, "tile copy must divide evenly");
 static_assert((BM * K_CPR) % NTHREADS == 0 && (BN * K_CPR) % NTHREADS == 0, "conv tile copy must divide evenly");
@@ -120,7 +134,7 @@ constexpr int OOB = 0x7fffffff;  // byte offset beyond any buffer: the load retu
 
 // The tile parameters appear as (otherwise unused) template arguments so that every configuration's
 // kernel has its own symbol name and a profiler lists configurations separately.
-template <bool CONV, int T_BM = BM, int T_BN = BN, int T_BK = BK, int T_WM = WAVE_M, int T_WN = WAVE_N>
+template <bool CONV, int T_BM = BM, int T_BN = BN, int T_BK = BK, int T_WM = WAVE_M, int T_WN = WAVE_N, int T_KG = KG>
 __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params p) {
     constexpr int LDA_S = Lds<CONV>::LDA, LDB_S = Lds<CONV>::LDB, A_STAGE = Lds<CONV>::A_STAGE, STAGE = Lds<CONV>::STAGE;
     extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -128,7 +142,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const int wave_kg = wave / WAVES_MN, wave_mn = wave % WAVES_MN;
+    const int wave_m = wave_mn / WAVES_N, wave_n = wave_mn % WAVES_N;
 
     // workgroup id -> tile: undo the round-robin deal over the 8 XCDs, then walk groups of tile rows
     const int ntiles = p.tiles_m * p.tiles_n;
@@ -275,8 +290,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 
     // MFMA 32x32x2: lane l supplies A[l % 32][l / 32] and B[l / 32][l % 32]
     const int frow = lane & 31, fk = lane >> 5;
-    const int a_rd = fk * LDA_S + wave_m * WAVE_M + frow;
-    const int b_rd = A_STAGE + fk * LDB_S + wave_n * WAVE_N + frow;
+    const int a_rd = (wave_kg * (BK / KG) + fk) * LDA_S + wave_m * WAVE_M + frow;
+    const int b_rd = A_STAGE + (wave_kg * (BK / KG) + fk) * LDB_S + wave_n * WAVE_N + frow;
 
     const int ktiles = (k_hi - k_lo + BK - 1) / BK;
     constexpr std::integral_constant<int, 0> set0{};
@@ -311,7 +326,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
 
         const float* sb = smem + SET * STAGE;
 #pragma unroll
-        for (int s = 0; s < BK / 2; s++) {
+        for (int s = 0; s < KSTEPS; s++) {
             float af[TM], bf[TN];
 #pragma unroll
             for (int i = 0; i < TM; i++) af[i] = sb[a_rd + s * 2 * LDA_S + i * 32];
@@ -328,7 +343,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
             // few instructions each (fragment reads are left to the scheduler, which keeps them a k step ahead)
             constexpr int MFMA = 0x008, VALU = 0x002, VALU_PER_MFMA = 3;
 #pragma unroll
-            for (int q = 0; q < (BK / 2) * TM * TN; q++) {
+            for (int q = 0; q < KSTEPS * TM * TN; q++) {
                 __builtin_amdgcn_sched_group_barrier(MFMA, 1, SET);
                 __builtin_amdgcn_sched_group_barrier(VALU, VALU_PER_MFMA, SET);
             }
@@ -344,6 +359,33 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
         tile(kt + 1, set1);
     }
     if (kt < ktiles) tile(kt, set0);
+
+    if (KG > 1) {
+        // every wave is past the last tile's barrier: the stages are free.  Groups 1.. leave their partial tiles
+        // in LDS ([group][wave tile][32x32 tile][register][lane]), group 0 adds them in group order and stores.
+        float* red = smem;
+        constexpr int TILE = TM * TN * 16 * 64;
+        if (wave_kg > 0) {
+            float* mine = red + ((wave_kg - 1) * WAVES_MN + wave_mn) * TILE + lane;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) mine[((i * TN + j) * 16 + v) * 64] = acc[i][j][v];
+        }
+        __syncthreads();
+        if (wave_kg > 0) return;
+        for (int g = 1; g < KG; g++) {
+            const float* theirs = red + ((g - 1) * WAVES_MN + wave_mn) * TILE + lane;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int v = 0; v < 16; v++) acc[i][j][v] += theirs[((i * TN + j) * 16 + v) * 64];
+        }
+    }
 
     // lane l holds column (l % 32); rows 8*(v/4) + 4*(l/32) + (v%4)
     const int col_l = lane & 31, row_l = (lane >> 5) * 4;
@@ -390,11 +432,11 @@ inline const char* info_json() {
         snprintf(buf, sizeof(buf),
                  "{\"family\": \"sgemm_f32\", \"arch\": \"gfx950\", \"mfma\": \"v_mfma_f32_32x32x2_f32\", "
                  "\"lds_stages\": 2, \"block_rows\": %d, \"block_cols\": %d, \"wave_rows\": %d, \"wave_cols\": %d, "
-                 "\"block_k\": %d, \"split_k\": \"up to 8 K partitions when the tiles leave compute units idle and the caller passes the workspace\", \"threads\": %d, \"lds_bytes\": %d, "
+                 "\"block_k\": %d, \"k_groups\": %d, \"split_k\": \"up to 8 K partitions when the tiles leave compute units idle and the caller passes the workspace\", \"threads\": %d, \"lds_bytes\": %d, "
                  "\"layout_a\": \"K x M row-major f32 (A transposed)\", \"layout_b\": \"K x N row-major f32\", "
                  "\"layout_c\": \"M x N row-major f32\", \"accumulate\": \"f32\", "
-                 "\"k_multiple\": 1, \"ld_multiple\": 4, \"conv\": \"NHWC x [OC][kH][kW][IC]; implicit GEMM when IC %% 4 == 0, else column buffer in the workspace\"}",
-                 BM, BN, WAVE_M, WAVE_N, BK, NTHREADS, LDS_BYTES);
+                 "\"k_multiple\": 1, \"ld_multiple\": 4, \"conv\": \"NHWC x [OC][kH][kW][IC]; implicit GEMM when IC %% 4 == 0, else channel-padded copies or a column buffer in the workspace\"}",
+                 BM, BN, WAVE_M, WAVE_N, BK, KG, NTHREADS, LDS_BYTES);
         done = true;
     }
     return buf;

@@ -408,7 +408,7 @@ def test_sgemm_f32_k_partitions():
     `helix_workspace_bytes` asks for (partial sums + fixed-order reduction), and run unpartitioned otherwise:
     both agree with the oracle, and on integer-valued inputs both are exact."""
     rng = np.random.default_rng(21)
-    for cfg in [(64, 64, 32, 32, 32), (128, 128, 16, 64, 64), (32, 32, 8, 32, 32)]:
+    for cfg in [(64, 64, 32, 32, 32), (128, 128, 16, 64, 64), (32, 32, 8, 32, 32), (32, 32, 64, 32, 32, 4)]:
         lib = load(b32.sgemm_library(*cfg))
         BM, BN, BK = cfg[:3]
         for (M, N, K) in [(100, 96, 2048), (257, 129, 1000), (64, 64, 8 * BK * 8), (300, 200, 137), (33, 500, 4096)]:
@@ -429,8 +429,9 @@ def test_sgemm_f32_k_partitions():
             assert np.array_equal(run_sgemm_f32(lib, Ai, Bi, False), exact), (cfg, M, N, K)
 
 
+# the last three are K-group configurations (2, 4 and 8 waves per 32 x 32 wave tile, partial tiles added in LDS)
 FP32_CONFIGS = [(128, 128, 16, 64, 64), (256, 128, 16, 128, 64), (32, 32, 8, 32, 32), (64, 256, 32, 32, 128),
-                (128, 64, 32, 64, 32)]
+                (128, 64, 32, 64, 32), (64, 64, 32, 32, 32, 2), (32, 64, 64, 32, 32, 4), (32, 32, 128, 32, 32, 8)]
 
 
 @pytest.mark.parametrize("cfg", FP32_CONFIGS)
@@ -480,7 +481,7 @@ def test_sgemm_f32_config1_and_large_k():
 
 
 def test_conv_f32_vs_oracle():
-    for cfg in [(128, 128, 16, 64, 64), (32, 32, 8, 32, 32), (64, 64, 32, 32, 32)]:
+    for cfg in [(128, 128, 16, 64, 64), (32, 32, 8, 32, 32), (64, 64, 32, 32, 32), (64, 32, 64, 32, 32, 4)]:
         lib = load(b32.sgemm_library(*cfg))
         for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS + CONV_GEOMS_ODD + [(2, 8, 8, 4, 8, 3, 3, 1, 1)]:
             x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW, dtype=np.float32)

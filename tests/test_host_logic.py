@@ -79,9 +79,18 @@ def test_fp32_template_space():
     for (BM, BN, BK, WM, WN) in cfgs:
         assert BM % WM == 0 and BN % WN == 0 and 32 <= BM <= 256 and 32 <= BN <= 256
         assert 64 * (BM // WM) * (BN // WN) <= 512
+    # K-group configurations: 32 x 32 wave tiles, K_GROUPS waves per tile, up to 1024 threads
+    kg = list(b32.iter_kgroup_configs())
+    assert len(kg) == 16 and len(set(kg)) == 16
+    for (BM, BN, BK, WM, WN, KG) in kg:
+        assert WM == WN == 32 and KG in (2, 4, 8) and (BK // 2) % KG == 0
+        assert 64 * (BM // WM) * (BN // WN) * KG <= 1024 and (KG - 1) * BM * BN * 4 <= 160 * 1024
     keys = p32.all_keys()
-    assert len(keys) == 143 + 6 and all(len(k) == 8 for k in keys)
-    assert b32.library_for_key((128, 64, 16, 64, 32, 2, 4, 4)).endswith("build/bin_fp32/libsgemm_128_64_16_64_32.so")
+    assert len(keys) == 143 + 16 + 6 and len(set(keys)) == len(keys) and all(len(k) == 8 for k in keys)
+    assert b32.config_key(64, 64, 16, 32, 32) == (64, 64, 16, 32, 32, 2, 1, 4)
+    assert b32.config_key(32, 32, 64, 32, 32, 4) == (32, 32, 64, 32, 32, 2, 4, 4)
+    assert b32.library_for_key((128, 64, 16, 64, 32, 2, 1, 4)).endswith("build/bin_fp32/libsgemm_128_64_16_64_32.so")
+    assert b32.library_for_key((64, 64, 64, 32, 32, 2, 4, 4)).endswith("build/bin_fp32/libsgemm_64_64_64_32_32_kg4.so")
     assert b32.library_for_key((4, 128, 0, 0, 0, 0, 4, 4)).endswith("build/bin_fp32/libgemv_fp32.so")
     assert b32.library_for_key((4, 128, 0, 0, 0, 1, 4, 4)).endswith("build/bin_fp32/libgemv_fp32_splitK.so")
 
@@ -133,10 +142,10 @@ def test_static_cost_models():
 
 def test_fp32_cost_model_hand_cases():
     K = p32.PROFILE_K
-    d = {(128, 128, 16, 64, 64, 2, 4, 4): 1.0, (256, 128, 16, 128, 64, 2, 4, 4): 1.8}
-    assert g32.cost_model(d, 4096, 4096, K) == (256, 128, 16, 128, 64, 2, 4, 4)
-    assert g32.cost_model(d, 300, 300, K) == (128, 128, 16, 64, 64, 2, 4, 4)
-    assert g32.config_cost((128, 128, 16, 64, 64, 2, 4, 4), 1.0, 4096, 4096, 2 * K) == pytest.approx(8.0)
+    d = {(128, 128, 16, 64, 64, 2, 1, 4): 1.0, (256, 128, 16, 128, 64, 2, 1, 4): 1.8}
+    assert g32.cost_model(d, 4096, 4096, K) == (256, 128, 16, 128, 64, 2, 1, 4)
+    assert g32.cost_model(d, 300, 300, K) == (128, 128, 16, 64, 64, 2, 1, 4)
+    assert g32.config_cost((128, 128, 16, 64, 64, 2, 1, 4), 1.0, 4096, 4096, 2 * K) == pytest.approx(8.0)
 
 
 def test_fp16_cost_model_two_point_profile():
@@ -182,7 +191,7 @@ def test_fp16_cost_model_two_point_profile():
 
 def test_fp32_cost_model_extra_points():
     K, Ks = p32.PROFILE_K, p32.PROFILE_K_SHORT
-    key = (64, 64, 16, 32, 32, 2, 4, 4)
+    key = (64, 64, 16, 32, 32, 2, 1, 4)
     d = helix_runtime.ProfDict({key: 30e-6})
     d.short, d.two_rounds, d.short_two_rounds = {key: 12e-6}, {key: 48e-6}, {key: 15e-6}
     pts = g32.extra_points(d, key)
@@ -191,13 +200,17 @@ def test_fp32_cost_model_extra_points():
     # one round of 256 tiles: the one-round line; 1024 x 1024 outputs with 64 x 64 tiles
     assert g32.config_cost(key, 30e-6, 1024, 1024, K, pts) == pytest.approx(30e-6)
     assert g32.config_cost(key, 30e-6, 1024, 1024, Ks, pts) == pytest.approx(12e-6)
-    # four rounds at the profile K: later rounds cost the two-round increment (18 us) or the minimum share of a
-    # lone round (30 us), whichever is larger
-    share = g32.later_round_min_share(K)
-    assert share == g32.LATER_ROUND_MIN_SHARE_SHORT and g32.later_round_min_share(4 * K) == g32.LATER_ROUND_MIN_SHARE_LONG
-    assert g32.config_cost(key, 30e-6, 2048, 2048, K, pts) == pytest.approx(30e-6 + 3 * max(18e-6, share * 30e-6))
-    # at the short K the increment (3 us) is below the share of a lone round (12 us), so the share applies
-    assert g32.config_cost(key, 30e-6, 2048, 2048, Ks, pts) == pytest.approx(12e-6 + 3 * share * 12e-6)
+    # four rounds at the profile K: later rounds cost the two-round increment (18 us), which is above what the
+    # matrix pipes need for a round (256 tiles x 64 x 64 x 1024 x 2 flop at 0.85 of 157.3 TFLOP/s = 16.1 us)
+    pipes = lambda kk: 2.0 * 256 * 64 * 64 * kk / (g32.LATER_ROUND_MFMA_FRACTION * g32.FP32_MFMA_FLOPS)
+    assert pipes(K) == pytest.approx(16.06e-6, rel=1e-3)
+    assert g32.config_cost(key, 30e-6, 2048, 2048, K, pts) == pytest.approx(30e-6 + 3 * 18e-6)
+    # at the short K the increment (3 us) is below the pipes' time for the round (4.0 us), which then applies
+    assert g32.config_cost(key, 30e-6, 2048, 2048, Ks, pts) == pytest.approx(12e-6 + 3 * pipes(Ks))
+    # BK = 32 over several rounds: 5 % on top
+    key32 = (64, 64, 32, 32, 32, 2, 1, 4)
+    assert g32.config_cost(key32, 30e-6, 2048, 2048, K, pts) == pytest.approx((30e-6 + 3 * 18e-6) * (1 + g32.BK32_MULTI_ROUND_COST))
+    assert g32.config_cost(key32, 30e-6, 1024, 1024, K, pts) == pytest.approx(30e-6)
     # a long problem on small tiles is bound by the rate the compute units take operands in
     big = g32.config_cost(key, 20e-6, 8192, 8192, 8192, (12e-6, 30e-6, 15e-6))
     assert big == pytest.approx(4.0 * 8192 ** 3 * (2 / 64) / g32.OPERAND_BYTES_PER_S)
@@ -310,8 +323,8 @@ def test_baseline_config_script_resolves_backend_functions():
         assert callable(be.gemm_result) and callable(be.gemm_oracle) and callable(be.conv_result)
     be16, be32 = bc.Backend("MI355X_FP16"), bc.Backend("MI355X_FP32")
     assert be16.is_gemv_key((0, 4, 128, 0, 0, 0, 0)) and not be16.is_gemv_key((2, 32, 64, 32, 32, 0, 128))
-    assert be32.is_gemv_key((4, 128, 0, 0, 0, 0, 4, 4)) and not be32.is_gemv_key((32, 64, 16, 32, 32, 2, 4, 4))
-    assert be16.block_rows((2, 32, 64, 32, 32, 0, 128)) == 32 and be32.block_rows((32, 64, 16, 32, 32, 2, 4, 4)) == 32
+    assert be32.is_gemv_key((4, 128, 0, 0, 0, 0, 4, 4)) and not be32.is_gemv_key((32, 64, 16, 32, 32, 2, 1, 4))
+    assert be16.block_rows((2, 32, 64, 32, 32, 0, 128)) == 32 and be32.block_rows((32, 64, 16, 32, 32, 2, 1, 4)) == 32
     assert set(bc.SECTIONS) == {"square", "gemv", "conv", "bert"}
     out = subprocess.run([sys.executable, os.path.join(ROOT, "helix_amd", "scripts", "benchmark_baseline_configs.py"),
                           "-c", "nothing"], capture_output=True, text=True,
