@@ -360,6 +360,41 @@ def test_conv_f16_baseline_layers_sampled():
         assert worst < TOL16 * scale, (batch, IC, H, W, OC, kH, kW, stride, pad)
 
 
+def _sampled_conv_check(y, x, w, stride, pad, tol, rng, n=40):
+    batch, H, W, IC = x.shape
+    OC, kH, kW, _ = w.shape
+    OH, OW = O.conv_out_hw(H, W, kH, kW, stride, pad)
+    assert y.shape == (batch, OH, OW, OC)
+    xp = np.zeros((batch, H + 2 * pad, W + 2 * pad, IC), np.float64)
+    xp[:, pad:pad + H, pad:pad + W] = x
+    w64 = w.astype(np.float64)
+    pts = [(0, 0, 0), (batch - 1, OH - 1, OW - 1), (batch - 1, 0, OW - 1), (0, OH - 1, 0)] + \
+          [(int(rng.integers(batch)), int(rng.integers(OH)), int(rng.integers(OW))) for _ in range(n)]
+    worst, scale = 0.0, 0.0
+    for (b, oh, ow) in pts:
+        patch = xp[b, oh * stride:oh * stride + kH, ow * stride:ow * stride + kW]
+        want = np.einsum("hwc,ohwc->o", patch, w64)
+        worst = max(worst, np.max(np.abs(y[b, oh, ow] - want)))
+        scale = max(scale, np.max(np.abs(want)))
+    assert not np.isnan(y).any()
+    assert worst < tol * scale, (x.shape, w.shape, stride, pad)
+
+
+def test_conv_first_layers_full_size_sampled():
+    """The three-channel first layers of AlexNet, GoogleNet and a VGG-style stem at batch 32 and 224 x 224 (the
+    channel-padded path at its real size, corners and image borders included): sampled output pixels against
+    float64, FP16 and FP32."""
+    rng = np.random.default_rng(12)
+    lib16 = load(b16.kernel_library("gemm", 2, 128, 64, 32, 32, 64))
+    lib32 = load(b32.sgemm_library(64, 64, 16, 32, 32))
+    for (batch, IC, H, W, OC, kH, kW, stride, pad) in [(32, 3, 224, 224, 96, 11, 11, 4, 0), (32, 3, 224, 224, 64, 7, 7, 2, 3),
+                                                       (32, 3, 224, 224, 64, 3, 3, 1, 1)]:
+        x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW)
+        _sampled_conv_check(run_conv(lib16, x, w, stride, pad, torch.float16), x, w, stride, pad, TOL16, rng)
+        x32, w32 = x.astype(np.float32), w.astype(np.float32)
+        _sampled_conv_check(run_conv(lib32, x32, w32, stride, pad, torch.float32), x32, w32, stride, pad, TOL32, rng)
+
+
 # ---------------------------------------------------------------------------------------------
 # vendor comparator libraries (rocBLAS behind the same C ABI)
 # ---------------------------------------------------------------------------------------------
