@@ -341,9 +341,12 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
         if (CONV) {
             // issue order of the block above: the index arithmetic of conv_offsets dealt out behind the MFMAs, a
             // few instructions each (fragment reads are left to the scheduler, which keeps them a k step ahead)
+            // (the first 16 MFMAs take all of it; asking for more groups only costs compile time, minutes for the
+            // 128 x 128 wave tile)
             constexpr int MFMA = 0x008, VALU = 0x002, VALU_PER_MFMA = 3;
+            constexpr int GROUPS = KSTEPS * TM * TN < 16 ? KSTEPS * TM * TN : 16;
 #pragma unroll
-            for (int q = 0; q < KSTEPS * TM * TN; q++) {
+            for (int q = 0; q < GROUPS; q++) {
                 __builtin_amdgcn_sched_group_barrier(MFMA, 1, SET);
                 __builtin_amdgcn_sched_group_barrier(VALU, VALU_PER_MFMA, SET);
             }
