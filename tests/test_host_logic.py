@@ -360,11 +360,12 @@ def test_every_built_library_exports_the_whole_abi():
         pytest.skip("kernel libraries are not built (run __graft_entry__.build())")
     want = set(_declared_symbols())
     # dlopen + dlsym only; no compute without a GPU.  A sample keeps this fast: every family, every 7th gemm
-    sample = [p for p in libs if "gemv" in p or "rocblas" in p] + libs[::7]
+    sample = [p for p in libs if "gemv" in p or "rocblas" in p or "miopen" in p] + [p for p in libs if "_kg" in p][::5] + libs[::7]
     for path in sample:
         assert set(hip_ctypes.exported_symbols(path)) == want, path
         info = hip_ctypes.HelixLib(path).info()
-        assert info["arch"] == "gfx950" and info["family"] in ("gemm_f16", "gemv_f16", "sgemm_f32", "gemv_f32", "rocblas_f16", "rocblas_f32")
+        assert info["arch"] == "gfx950" and info["family"] in ("gemm_f16", "gemv_f16", "sgemm_f32", "gemv_f32", "rocblas_f16", "rocblas_f32",
+                                                           "miopen")
 
 
 def test_all_expected_libraries_are_built():
@@ -387,3 +388,7 @@ def test_info_matches_file_name():
     assert (info["k_stages"], info["block_rows"], info["block_cols"], info["wave_rows"], info["wave_cols"],
             info["block_k"], info["split_k"]) == (2, 256, 128, 64, 64, 64, 1)
     assert info["threads"] == 64 * 4 * 2 and info["lds_bytes"] == 2 * (256 + 128) * 64 * 2
+    # a K-group configuration: 4 waves on the one 32 x 32 wave tile
+    info = hip_ctypes.HelixLib(b32.sgemm_library(32, 32, 64, 32, 32, 4)).info()
+    assert (info["block_rows"], info["block_cols"], info["block_k"], info["k_groups"], info["threads"]) == (32, 32, 64, 4, 256)
+    assert hip_ctypes.HelixLib(b32.sgemm_library(64, 64, 16, 32, 32)).info()["k_groups"] == 1
