@@ -8,15 +8,16 @@
 // Role in the reference: src_template/Ampere_FP32/sgemm.cu:97-350 (`mySgemmCPAsyncTemplate`, a CUDA-core
 // register-tiled SGEMM with macros BM, BN, BK, TM, TN, :60-93).  Here the contraction runs on
 // v_mfma_f32_32x32x2_f32: one wave64 owns a WAVE_M x WAVE_N tile made of 32x32 MFMA tiles, each MFMA
-// consuming two k values; products are accumulated in ascending k, the same order the CPU path uses.
+// consuming two k values; products are accumulated in ascending k within a K partition, the order the CPU
+// path uses.
 //
-// Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N.
+// Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N, K_GROUPS
+// (waves per wave tile, each taking BK / K_GROUPS of every K tile; 1 unless the configuration is a K-group one).
 //
 // K partitions: a problem with fewer than 576 output tiles and a long K is split along K over blockIdx.y, up
-// to 8 ways (at least 768 of K each, 256 when there are at most 128 tiles, 64 at most 32); partial sums go to the
-// caller's workspace
-// (helix_workspace_bytes) and a second kernel adds them in partition order.  Without the workspace the
-// problem runs unpartitioned.  The reference's FP32 template has no K partition.
+// to 8 ways (at least 768 of K each, 256 when there are at most 128 tiles, 64 at most 32); partial sums go to
+// the caller's workspace (helix_workspace_bytes) and a second kernel adds them in partition order.  Without
+// the workspace the problem runs unpartitioned.  The reference's FP32 template has no K partition.
 //
 // LDS layout: A stage is [BK][BM + 32] floats, B stage [BK][BN + 32]; a fragment read takes lanes 0-31
 // from row k and lanes 32-63 from row k+1, and the 32-float row padding puts the two half-waves on
