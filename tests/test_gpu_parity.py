@@ -380,6 +380,57 @@ def _sampled_conv_check(y, x, w, stride, pad, tol, rng, n=40):
     assert worst < tol * scale, (x.shape, w.shape, stride, pad)
 
 
+def test_gemm_random_shapes_vs_oracle():
+    """Seeded random GEMM extents (ragged M and N, K from 1 to a few thousand so that K partitions of every
+    size occur) on tile, split-K, K-group and GEMV libraries, FP16 and FP32, against the oracle."""
+    rng = np.random.default_rng(44)
+    lib16 = [load(b16.kernel_library("gemm", 2, 128, 96, 64, 48, 128)), load(b16.kernel_library("gemm_splitK", 2, 64, 64, 32, 32, 64)),
+             load(b16.kernel_library("gemm_splitK", 2, 32, 128, 32, 32, 128))]
+    lib32 = [load(b32.sgemm_library(128, 64, 32, 64, 32)), load(b32.sgemm_library(32, 32, 32, 32, 32, 4)),
+             load(b32.sgemm_library(64, 32, 128, 32, 32, 8))]
+    gemv16, gemv32 = load(b16.kernel_library("gemv")), load(b32.kernel_library("gemv_fp32"))
+    for case in range(36):
+        M, N = int(rng.integers(1, 400)), int(rng.integers(1, 400))
+        K = int(rng.choice([1, 7, 33, 250, 1000, 2500])) + int(rng.integers(0, 40))
+        A = seeded_inputs.uniform_pm1((M, K), seeded_inputs.SEED_A + case)
+        B = seeded_inputs.uniform_pm1((K, N), seeded_inputs.SEED_B + case)
+        A16, B16 = A.astype(np.float16), B.astype(np.float16)
+        got = run_gemm_f16(lib16[case % 3], A16, B16)
+        assert not np.isnan(got).any() and normwise(got, O.hgemm_f32acc(A16, B16)) < TOL16, (case, M, N, K)
+        got = run_sgemm_f32(lib32[case % 3], A, B)
+        assert not np.isnan(got).any() and normwise(got, O.sgemm_seqk(A, B)) < TOL32, (case, M, N, K)
+        if M <= 16:
+            got = run_gemm_f16(gemv16, A16, B16)
+            assert not np.isnan(got).any() and normwise(got, O.hgemm_f32acc(A16, B16)) < TOL16, (case, M, N, K)
+
+
+def test_conv_random_geometries_vs_oracle():
+    """Seeded random small convolutions, channel counts 1 ... 20 (implicit gather, channel-padded copies and
+    column-buffer paths all occur), strides 1 ... 3, padding up to the filter size, rectangular images and
+    filters: FP16 and FP32 against the oracle."""
+    rng = np.random.default_rng(33)
+    lib16 = [load(b16.kernel_library("gemm", 2, 64, 64, 32, 32, 64)), load(b16.kernel_library("gemm_splitK", 2, 128, 64, 64, 32, 128))]
+    lib32 = [load(b32.sgemm_library(64, 64, 16, 32, 32)), load(b32.sgemm_library(32, 64, 64, 32, 32, 4))]
+    for case in range(40):
+        IC = int(rng.integers(1, 21))
+        kH, kW = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        stride, pad = int(rng.integers(1, 4)), int(rng.integers(0, max(kH, kW)))
+        H, W = int(rng.integers(kH, kH + 12)), int(rng.integers(kW, kW + 12))
+        batch, OC = int(rng.integers(1, 4)), int(rng.integers(1, 41))
+        if (H + 2 * pad - kH) // stride + 1 < 1 or (W + 2 * pad - kW) // stride + 1 < 1:
+            continue
+        x, w = seeded_inputs.conv_operands(batch, IC, H, W, OC, kH, kW)
+        want = O.conv2d_nhwc(x, w, stride, pad)
+        geom = (case, batch, H, W, IC, OC, kH, kW, stride, pad)
+        got = run_conv(lib16[case % 2], x, w, stride, pad, torch.float16)
+        assert got.shape == want.shape and not np.isnan(got).any(), geom
+        assert normwise(got, want) < TOL16, geom
+        x32, w32 = x.astype(np.float32), w.astype(np.float32)
+        got = run_conv(lib32[case % 2], x32, w32, stride, pad, torch.float32)
+        assert got.shape == want.shape and not np.isnan(got).any(), geom
+        assert normwise(got, O.conv2d_nhwc(x32, w32, stride, pad)) < TOL32, geom
+
+
 def test_conv_first_layers_full_size_sampled():
     """The three-channel first layers of AlexNet, GoogleNet and a VGG-style stem at batch 32 and 224 x 224 (the
     channel-padded path at its real size, corners and image borders included): sampled output pixels against
