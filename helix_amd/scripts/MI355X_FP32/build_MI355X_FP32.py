@@ -45,7 +45,7 @@ def is_valid_config(BMt, BNt, BM, BN, BK=16, WAVE_M=64, WAVE_N=64, KG=1):
         return False
     if (BM * BK // 4) % threads or (BN * BK // 4) % threads:       # conv tile copy, 16-byte chunks along K
         return False
-    conv_pad = 32 + 64 // BK          # LDS row padding of the convolution mode, the wider of the two
+    conv_pad = 32 + max(64 // BK, 1)  # LDS row padding of the convolution mode, the wider of the two
     if 2 * BK * (BM + conv_pad + BN + conv_pad) * 4 > LDS_LIMIT:
         return False
     if WAVE_M * WAVE_N // 64 > 256:

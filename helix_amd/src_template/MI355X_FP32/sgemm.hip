@@ -76,8 +76,9 @@ constexpr int KSTEPS = BK / 2 / KG;   // MFMA k steps (2 of K each) of one wave 
 // LDS row strides in floats.  GEMM mode: +32, which puts the two half-waves of a fragment read on different bank
 // halves and keeps rows 16-byte aligned for the 128-bit tile writes.  CONV mode writes scalars, BK/4 lanes per
 // tile row along k: the extra 16 / (BK/4) floats make the rows those lanes write fall on different banks
-// (4 * stride = 64 / (BK/4) mod 64) instead of all on one.
-constexpr int CONV_PAD = 32 + (BK >= 8 ? 64 / BK : 0);
+// (4 * stride = 64 / (BK/4) mod 64) instead of all on one; from BK = 64 on one extra float (an odd stride: 16
+// distinct banks for the 16 or 32 lanes of a row, where an even one put them all on the same bank).
+constexpr int CONV_PAD = 32 + (BK >= 64 ? 1 : BK >= 8 ? 64 / BK : 0);
 template <bool CONV> struct Lds {
     static constexpr int LDA = BM + (CONV ? CONV_PAD : 32), LDB = BN + (CONV ? CONV_PAD : 32);
     static constexpr int A_STAGE = BK * LDA, B_STAGE = BK * LDB;    // floats

@@ -387,7 +387,7 @@ def test_gemm_random_shapes_vs_oracle():
     lib16 = [load(b16.kernel_library("gemm", 2, 128, 96, 64, 48, 128)), load(b16.kernel_library("gemm_splitK", 2, 64, 64, 32, 32, 64)),
              load(b16.kernel_library("gemm_splitK", 2, 32, 128, 32, 32, 128))]
     lib32 = [load(b32.sgemm_library(128, 64, 32, 64, 32)), load(b32.sgemm_library(32, 32, 32, 32, 32, 4)),
-             load(b32.sgemm_library(64, 32, 128, 32, 32, 8))]
+             load(b32.sgemm_library(32, 32, 128, 32, 32, 8))]
     gemv16, gemv32 = load(b16.kernel_library("gemv")), load(b32.kernel_library("gemv_fp32"))
     for case in range(36):
         M, N = int(rng.integers(1, 400)), int(rng.integers(1, 400))

@@ -81,12 +81,12 @@ def test_fp32_template_space():
         assert 64 * (BM // WM) * (BN // WN) <= 512
     # K-group configurations: 32 x 32 wave tiles, K_GROUPS waves per tile, up to 1024 threads
     kg = list(b32.iter_kgroup_configs())
-    assert len(kg) == 16 and len(set(kg)) == 16
+    assert len(kg) == 14 and len(set(kg)) == 14
     for (BM, BN, BK, WM, WN, KG) in kg:
         assert WM == WN == 32 and KG in (2, 4, 8) and (BK // 2) % KG == 0
         assert 64 * (BM // WM) * (BN // WN) * KG <= 1024 and (KG - 1) * BM * BN * 4 <= 160 * 1024
     keys = p32.all_keys()
-    assert len(keys) == 143 + 16 + 6 and len(set(keys)) == len(keys) and all(len(k) == 8 for k in keys)
+    assert len(keys) == 143 + 14 + 6 and len(set(keys)) == len(keys) and all(len(k) == 8 for k in keys)
     assert b32.config_key(64, 64, 16, 32, 32) == (64, 64, 16, 32, 32, 2, 1, 4)
     assert b32.config_key(32, 32, 64, 32, 32, 4) == (32, 32, 64, 32, 32, 2, 4, 4)
     assert b32.library_for_key((128, 64, 16, 64, 32, 2, 1, 4)).endswith("build/bin_fp32/libsgemm_128_64_16_64_32.so")
