@@ -32,23 +32,42 @@ BK32_MULTI_ROUND_COST = 0.05
 OPERAND_BYTES_PER_S = 6.5e12
 
 
-SPLITK_MAX, SPLITK_TARGET, SPLITK_MIN_K = 8, 768, 768   # as in src_template/MI355X_FP32/sgemm.hip
+SPLITK_MAX, SPLITK_TARGET = 8, 768   # as in src_template/MI355X_FP32/sgemm.hip
 SPLITK_MIN_K_FEW, SPLITK_FEW_TILES = 256, 128
 SPLITK_MIN_K_TINY, SPLITK_TINY_TILES = 64, 32
+SPLITK_MFMA_FRACTION, SPLITK_REDUCE_BYTES_PER_S, SPLITK_MIN_GAIN, SPLITK_MIN_K_BALANCE = 0.8, 5e12, 0.98, 128
 SPLITK_REDUCE_LAUNCH_S = 4e-6   # the reduction kernel of a K-partitioned launch
 
 
 def split_factor(k, M, N, K):
-    """K partitions the SGEMM libraries use for this problem (same rule as their host side): when the tiles give
-    fewer than three quarters of SPLITK_TARGET workgroups, as many as reach the target, at most SPLITK_MAX, at
-    least SPLITK_MIN_K of K per partition (SPLITK_MIN_K_FEW when there are at most SPLITK_FEW_TILES tiles)."""
+    """K partitions the SGEMM libraries use for this problem (same rule, same arithmetic as their host side).  At
+    most SPLITK_FEW_TILES tiles: as many as reach SPLITK_TARGET workgroups, at most SPLITK_MAX, at least
+    SPLITK_MIN_K_FEW of K per partition (SPLITK_MIN_K_TINY up to SPLITK_TINY_TILES tiles).  More tiles: the count
+    that makes rounds of 256 workgroups x one partition's K walk, plus a fixed cost per workgroup and the
+    reduction pass, smallest."""
     if k[2] == 0:
         return 1
-    tiles = math.ceil(M / k[0]) * math.ceil(N / k[1])
-    if tiles <= 0 or tiles >= SPLITK_TARGET * 3 // 4:
+    BM, BN, BK = k[0], k[1], k[2]
+    tiles = math.ceil(M / BM) * math.ceil(N / BN)
+    if tiles <= 0:
         return 1
-    min_k = SPLITK_MIN_K_TINY if tiles <= SPLITK_TINY_TILES else SPLITK_MIN_K_FEW if tiles <= SPLITK_FEW_TILES else SPLITK_MIN_K
-    return max(min(math.ceil(SPLITK_TARGET / tiles), SPLITK_MAX, K // min_k), 1)
+    if tiles <= SPLITK_FEW_TILES:
+        min_k = SPLITK_MIN_K_TINY if tiles <= SPLITK_TINY_TILES else SPLITK_MIN_K_FEW
+        return max(min(math.ceil(SPLITK_TARGET / tiles), SPLITK_MAX, K // min_k), 1)
+    per_k = 2.0 * BM * BN * NUM_CU / (SPLITK_MFMA_FRACTION * FP32_MFMA_FLOPS)
+    fixed = 1e-6 + 1.5e-6 * (BM * BN) / (128.0 * 128.0)
+    ktiles = (K + BK - 1) // BK
+    best, best_t = 1, 0.0
+    s = 1
+    while s <= SPLITK_MAX and (s == 1 or K // s >= SPLITK_MIN_K_BALANCE):
+        walk = float(((ktiles + s - 1) // s) * BK)
+        rounds = float((tiles * s + NUM_CU - 1) // NUM_CU)
+        reduce = SPLITK_REDUCE_LAUNCH_S + (s + 1.0) * float(M) * float(N) * 4.0 / SPLITK_REDUCE_BYTES_PER_S if s > 1 else 0.0
+        t = rounds * (walk * per_k + fixed) + reduce
+        if s == 1 or t < best_t * SPLITK_MIN_GAIN:
+            best, best_t = s, t
+        s += 1
+    return best
 
 
 def _line(x0, y0, x1, y1, x):

@@ -14,10 +14,11 @@
 // Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N, K_GROUPS
 // (waves per wave tile, each taking BK / K_GROUPS of every K tile; 1 unless the configuration is a K-group one).
 //
-// K partitions: a problem with fewer than 576 output tiles and a long K is split along K over blockIdx.y, up
-// to 8 ways (at least 768 of K each, 256 when there are at most 128 tiles, 64 at most 32); partial sums go to
-// the caller's workspace (helix_workspace_bytes) and a second kernel adds them in partition order.  Without
-// the workspace the problem runs unpartitioned.  The reference's FP32 template has no K partition.
+// K partitions: a problem is split along K over blockIdx.y, up to 8 ways, when that shortens the launch: few
+// tiles and a long K (compute units idle), or a tile count that leaves the last round of workgroups mostly
+// empty (split_factor below); partial sums go to the caller's workspace (helix_workspace_bytes) and a second
+// kernel adds them in partition order.  Without the workspace the problem runs unpartitioned.  The
+// reference's FP32 template has no K partition.
 //
 // LDS layout: A stage is [BK][BM + 32] floats, B stage [BK][BN + 32]; a fragment read takes lanes 0-31
 // from row k and lanes 32-63 from row k+1, and the 32-float row padding puts the two half-waves on
@@ -447,27 +448,51 @@ inline const char* info_json() {
     return buf;
 }
 
-// K partitions for an M x N x K problem: when the tiles alone give fewer than three quarters of SPLITK_TARGET
-// workgroups (three per compute unit: this kernel hides its LDS and global latencies across workgroups that share
-// a compute unit, and a launch of one to two rounds of tiles leaves most units with one), as many as reach
-// the target, at most SPLITK_MAX, and never so many that a partition walks less than SPLITK_MIN_K of K
-// (SPLITK_MIN_K_FEW when the tiles do not even cover half of the compute units, SPLITK_MIN_K_TINY when there are
-// at most 32 of them: a 14 x 14 x 480 -> 192 1x1 convolution went 18 -> 10 us).
-// Measured on 1521 x 768 x 2304: 83 us unpartitioned, 62 us three-way.  The reference's FP32 template has no K
-// partition (src_template/Ampere_FP32/sgemm.cu); its FP16 one is 2-way (gemm_splitK.cu:124-129).
-constexpr int SPLITK_MAX = 8, SPLITK_TARGET = SPLITK_TARGET_BLOCKS, SPLITK_MAX_TILES = SPLITK_TARGET * 3 / 4,
-              SPLITK_MIN_K = 768, SPLITK_MIN_K_FEW = 256, SPLITK_FEW_TILES = 128, SPLITK_MIN_K_TINY = 64,
-              SPLITK_TINY_TILES = 32;
+// K partitions for an M x N x K problem.  At most SPLITK_FEW_TILES tiles (they do not even cover half of the
+// compute units): towards SPLITK_TARGET workgroups, three per compute unit -- this kernel hides its LDS and
+// global latencies across workgroups that share a compute unit --, at most SPLITK_MAX, and never so many that a
+// partition walks less than SPLITK_MIN_K_FEW of K (SPLITK_MIN_K_TINY when there are at most 32 tiles: a
+// 14 x 14 x 480 -> 192 1x1 convolution went 18 -> 10 us).  The reference's FP32 template has no K partition
+// (src_template/Ampere_FP32/sgemm.cu); its FP16 one is 2-way (gemm_splitK.cu:124-129).
+constexpr int SPLITK_MAX = 8, SPLITK_TARGET = SPLITK_TARGET_BLOCKS, SPLITK_MIN_K_FEW = 256, SPLITK_FEW_TILES = 128,
+              SPLITK_MIN_K_TINY = 64, SPLITK_TINY_TILES = 32;
+
+// More than SPLITK_FEW_TILES tiles: workgroups beyond one per compute unit queue up behind each other, so a launch
+// takes ceil(workgroups / 256) rounds of one partition's K walk, and the partition count is the one that makes
+// rounds x walk (plus a fixed cost per workgroup and the reduction pass) smallest -- 196 tiles of K = 4608 take four
+// rounds of 1152 four ways and four rounds of 922 five ways (measured 305 -> 262 us), 784 tiles four rounds of 4608
+// unpartitioned and thirteen of 1152 four ways (1060 -> 938 us).  Times in seconds, matrix pipes at
+// SPLITK_MFMA_FRACTION of their peak; scripts/MI355X_FP32/MI355X_FP32_gemm.py evaluates the same expression.
+constexpr double SPLITK_MFMA_FRACTION = 0.8, SPLITK_FP32_MFMA_FLOPS = 157.3e12, SPLITK_REDUCE_BYTES_PER_S = 5e12,
+                 SPLITK_REDUCE_LAUNCH_S = 4e-6, SPLITK_MIN_GAIN = 0.98;
+constexpr int SPLITK_MIN_K_BALANCE = 128, SPLITK_COMPUTE_UNITS = 256;
 
 inline int split_factor(long long M, long long N, long long K) {
     const long long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    if (tiles <= 0 || tiles >= SPLITK_MAX_TILES) return 1;
-    long long s = (SPLITK_TARGET + tiles - 1) / tiles;
-    if (s > SPLITK_MAX) s = SPLITK_MAX;
-    const long long min_k = tiles <= SPLITK_TINY_TILES ? SPLITK_MIN_K_TINY
-                            : tiles <= SPLITK_FEW_TILES ? SPLITK_MIN_K_FEW : SPLITK_MIN_K;
-    if (s > K / min_k) s = K / min_k;
-    return s < 1 ? 1 : (int)s;
+    if (tiles <= 0) return 1;
+    if (tiles <= SPLITK_FEW_TILES) {
+        long long s = (SPLITK_TARGET + tiles - 1) / tiles;
+        if (s > SPLITK_MAX) s = SPLITK_MAX;
+        const long long min_k = tiles <= SPLITK_TINY_TILES ? SPLITK_MIN_K_TINY : SPLITK_MIN_K_FEW;
+        if (s > K / min_k) s = K / min_k;
+        return s < 1 ? 1 : (int)s;
+    }
+    const double per_k = 2.0 * BM * BN * SPLITK_COMPUTE_UNITS / (SPLITK_MFMA_FRACTION * SPLITK_FP32_MFMA_FLOPS);
+    const double fixed = 1e-6 + 1.5e-6 * (BM * BN) / (128.0 * 128.0);
+    const long long ktiles = (K + BK - 1) / BK;
+    int best = 1;
+    double best_t = 0.0;
+    for (int s = 1; s <= SPLITK_MAX && (s == 1 || K / s >= SPLITK_MIN_K_BALANCE); s++) {
+        const double walk = (double)(((ktiles + s - 1) / s) * BK);
+        const double rounds = (double)((tiles * s + SPLITK_COMPUTE_UNITS - 1) / SPLITK_COMPUTE_UNITS);
+        const double reduce = s > 1 ? SPLITK_REDUCE_LAUNCH_S + (s + 1.0) * (double)M * (double)N * 4.0 / SPLITK_REDUCE_BYTES_PER_S : 0.0;
+        const double t = rounds * (walk * per_k + fixed) + reduce;
+        if (s == 1 || t < best_t * SPLITK_MIN_GAIN) {   // a further partition has to pay for itself
+            best_t = t;
+            best = s;
+        }
+    }
+    return best;
 }
 
 // Partial sums of the K partitions; a caller that passes less runs the problem unpartitioned.

@@ -21,6 +21,7 @@ from utils.helix_runtime import load
 from utils.hip_ctypes import HelixError, HELIX_ERR_INVALID_VALUE, HELIX_ERR_UNSUPPORTED, HELIX_ERR_WORKSPACE
 from MI355X_FP16 import build_MI355X_FP16 as b16
 from MI355X_FP32 import build_MI355X_FP32 as b32
+from MI355X_FP32 import MI355X_FP32_gemm as g32
 
 pytestmark = pytest.mark.gpu
 
@@ -497,9 +498,10 @@ def test_sgemm_f32_k_partitions():
     for cfg in [(64, 64, 32, 32, 32), (128, 128, 16, 64, 64), (32, 32, 8, 32, 32), (32, 32, 64, 32, 32, 4)]:
         lib = load(b32.sgemm_library(*cfg))
         BM, BN, BK = cfg[:3]
-        for (M, N, K) in [(100, 96, 2048), (257, 129, 1000), (64, 64, 8 * BK * 8), (300, 200, 137), (33, 500, 4096)]:
-            tiles = -(-M // BM) * -(-N // BN)
-            want_splits = 1 if tiles >= 576 else max(min(-(-768 // tiles), 8, K // (64 if tiles <= 32 else 256 if tiles <= 128 else 768)), 1)
+        for (M, N, K) in [(100, 96, 2048), (257, 129, 1000), (64, 64, 8 * BK * 8), (300, 200, 137), (33, 500, 4096),
+                          (1000, 640, 900), (1500, 768, 2304)]:
+            # the host scripts mirror the library's partition rule; the two must agree for the workspace to fit
+            want_splits = g32.split_factor(b32.config_key(*cfg), M, N, K)
             assert lib.workspace_bytes(M, N, K) == (want_splits * M * N * 4 if want_splits > 1 else 0), (cfg, M, N, K)
             A = seeded_inputs.uniform_pm1((M, K), seeded_inputs.SEED_A)
             B = seeded_inputs.uniform_pm1((K, N), seeded_inputs.SEED_B)

@@ -189,6 +189,21 @@ def test_fp16_cost_model_two_point_profile():
         pytest.approx(g16.GEMV_LAUNCH_FLOOR_S + g16.GEMV_SPLITK_EXTRA_S)
 
 
+def test_fp32_split_factor_rule():
+    key = (128, 128, 16, 32, 64, 2, 1, 4)
+    # few tiles: towards 768 workgroups, at most 8, at least 256 (64 up to 32 tiles) of K per partition
+    assert g32.split_factor(key, 1024, 1024, 1024) == 4          # 64 tiles
+    assert g32.split_factor(key, 256, 256, 4096) == 8            # 4 tiles
+    assert g32.split_factor(key, 256, 256, 200) == 3
+    # more than 128 tiles: rounds of 256 workgroups x K walk; 196 tiles go five ways (four rounds of 922 instead of
+    # four of 1152), 256 tiles stay whole, 784 tiles go three ways
+    assert g32.split_factor(key, 6272, 512, 4608) == 5
+    assert g32.split_factor(key, 2048, 2048, 2048) == 1
+    assert g32.split_factor(key, 25088, 512, 4608) == 3
+    assert g32.split_factor((64, 64, 32, 32, 32, 2, 1, 4), 1024, 1024, 1024) == 1
+    assert g32.split_factor((4, 128, 0, 0, 0, 0, 4, 4), 4, 4096, 4096) == 1    # GEMV rows never partition here
+
+
 def test_fp32_cost_model_extra_points():
     K, Ks = p32.PROFILE_K, p32.PROFILE_K_SHORT
     key = (64, 64, 16, 32, 32, 2, 1, 4)
