@@ -27,7 +27,9 @@ def _find_include_dir():
 
 HIPCC = os.environ.get("HIPCC", "hipcc")
 # -packed-fp32-ops is switched off on purpose: the compiler must not form packed FP32 VALU ops here.
-COMPILE_OPTIONS = ("-O3 -std=c++17 --offload-arch=gfx950 -shared -fPIC -w "
+# Hidden visibility + -Bsymbolic: a library exports the helix_* entry points of include/helix_abi.h and nothing
+# else, and its own calls bind inside it, so several configurations can share a process however they are opened.
+COMPILE_OPTIONS = ("-O3 -std=c++17 --offload-arch=gfx950 -shared -fPIC -w -fvisibility=hidden -Wl,-Bsymbolic "
                    "-Xclang -target-feature -Xclang -packed-fp32-ops")
 
 

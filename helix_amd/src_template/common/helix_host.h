@@ -36,6 +36,7 @@
     } while (0)
 
 namespace helix_host {
+namespace {   // internal linkage: a library exports the helix_* entry points only
 
 // Deterministic fill: value = scale * u, u in [-1, 1) from an integer hash of the element index.
 __global__ void fill_f16_kernel(_Float16* p, size_t n, float scale, uint32_t seed) {
@@ -115,6 +116,7 @@ int time_launches(Launch&& launch, hipStream_t s, int warmup, int iters, double*
     return 0;
 }
 
+}  // namespace
 }  // namespace helix_host
 
 extern "C" {

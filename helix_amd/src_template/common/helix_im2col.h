@@ -25,6 +25,7 @@
 #include "helix_fastdiv.h"
 
 namespace helix_im2col {
+namespace {   // internal linkage: every template library carries its own copy and exports none of it
 
 using helix_fastdiv::FastDiv;
 
@@ -58,7 +59,9 @@ template <typename T, int VEC>
 __global__ void im2col_rows_kernel(const T* x, T* col, Geom g, int ldk, FastDiv by_chunks) {
     const int chunks = by_chunks.d;
     const int total = g.M * chunks;
-    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+    // the running index is 64-bit: total may lie within one grid stride of 2^31, where a 32-bit index would wrap
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+        const int idx = (int)i;
         const int m = by_chunks.div(idx), k0 = (idx - m * chunks) * VEC;
         const Pixel px = pixel_of(g, m);
         int f = g.by_IC.div(k0);
@@ -133,7 +136,8 @@ template <typename T, int VEC>
 __global__ void pad_channels_kernel(const T* src, T* dst, int rows, int IC, int ICp, FastDiv by_chunks) {
     const int chunks = by_chunks.d;
     const int total = rows * chunks;
-    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+        const int idx = (int)i;
         const int r = by_chunks.div(idx), c0 = (idx - r * chunks) * VEC;
         const T* from = src + (size_t)r * IC + c0;
         struct alignas(sizeof(T) * VEC) Chunk { T v[VEC]; } chunk;
@@ -160,4 +164,5 @@ inline int grid_for(size_t total) {
 
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
+}  // namespace
 }  // namespace helix_im2col

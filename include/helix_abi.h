@@ -41,6 +41,11 @@
 extern "C" {
 #endif
 
+/* Only the entry points below are exported; everything else in a template library has hidden visibility
+ * (the libraries are built with -fvisibility=hidden -Wl,-Bsymbolic), so two configurations can live in one
+ * process, however they are opened, without binding to each other's tile code. */
+#define HELIX_API __attribute__((visibility("default")))
+
 #define HELIX_OK 0
 #define HELIX_ERR_INVALID_VALUE 1 /* same value as hipErrorInvalidValue */
 #define HELIX_ERR_UNSUPPORTED 801 /* same value as hipErrorNotSupported */
@@ -51,18 +56,18 @@ extern "C" {
  * Returns the number of bytes needed including the NUL; if that exceeds `cap` nothing is written.
  * Replaces: the configuration encoded in the reference's executable names
  * (scripts/Ampere_FP16/build_Ampere_FP16.py:13-27, scripts/Ampere_FP32/build_Ampere_FP32.py:18). */
-int helix_info(char* json, int cap);
+HELIX_API int helix_info(char* json, int cap);
 
 /* Bytes of device scratch `helix_gemm` needs for this shape (0 unless the template splits K).
  * Replaces: nothing -- the reference's split-K accumulates with FP16 atomics into C
  * (src_template/Ampere_FP16/gemm_splitK.cu:495-506); here partial sums go through an FP32 workspace. */
-size_t helix_workspace_bytes(int M, int N, int K);
+HELIX_API size_t helix_workspace_bytes(int M, int N, int K);
 
 /* One GEMM / GEMV launch on `stream`.  lda/ldb/ldc are row strides in elements.
  * Replaces: the launchers `void f(half*, half*, half*, int M, int N, int K)`
  * (src_template/Ampere_FP16/gemm.cu:551-565, gemv.cu:218-252, gemv_splitK.cu:224-260) and
  * `mySgemmCPAsyncTemplate<<<>>>(a, b, c, M, N, K)` (src_template/Ampere_FP32/sgemm.cu:97,634). */
-int helix_gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
+HELIX_API int helix_gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
                void* workspace, size_t workspace_bytes, void* stream);
 
 /* Bytes of device scratch `helix_conv2d` needs for this problem: the split-K partial sums of the implicit
@@ -71,25 +76,25 @@ int helix_gemm(const void* A, const void* B, void* C, int M, int N, int K, int l
  * weights of the explicit im2col path.
  * Replaces: the `col` buffer the reference's im2col executable allocates for itself
  * (src_template/Ampere_FP16/im2col.cu:140-150). */
-size_t helix_conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad);
+HELIX_API size_t helix_conv_workspace_bytes(int batch, int H, int W, int IC, int OC, int kH, int kW, int stride, int pad);
 
 /* One NHWC convolution on `stream`: implicit GEMM (no column buffer) when IC is a multiple of the gather
  * chunk; else the same on copies with the channels zero-padded to the chunk, or (IC = 1; 2 in FP16) im2col
  * into the workspace followed by the GEMM, as the reference does for every layer.
  * Replaces: `im2col batch IC H W OC kH kW stride pad` followed by the GEMM executable
  * (scripts/Ampere_FP16/Ampere_FP16_conv.py:431-446, src_template/Ampere_FP16/im2col.cu:38-97). */
-int helix_conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
+HELIX_API int helix_conv2d(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
                  int kW, int stride, int pad, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Times caller-owned buffers: `warmup` untimed launches, then `iters` launches between two HIP
  * events recorded on `stream`; *avg_s = elapsed / iters in seconds.
  * Replaces: the event-timed loop of testF16F16GemmPerformance
  * (src_template/Ampere_FP16/gemm.cu:636-652) for callers that bring their own data. */
-int helix_gemm_timed(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
+HELIX_API int helix_gemm_timed(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
                      void* workspace, size_t workspace_bytes, void* stream, int warmup, int iters,
                      double* avg_s);
 
-int helix_conv2d_timed(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
+HELIX_API int helix_conv2d_timed(const void* x, const void* w, void* y, int batch, int H, int W, int IC, int OC, int kH,
                        int kW, int stride, int pad, void* workspace, size_t workspace_bytes, void* stream,
                        int warmup, int iters, double* avg_s);
 
@@ -102,12 +107,12 @@ int helix_conv2d_timed(const void* x, const void* w, void* y, int batch, int H, 
  * `gemm_... M N K` whose stdout the profiler parses (src_template/Ampere_FP16/gemm.cu:622-692,
  * gemv.cu:320-435, src_template/Ampere_FP32/sgemm.cu:427-466,568-657;
  * scripts/Ampere_FP16/profile_Ampere_FP16.py:36-38). */
-int helix_bench(int M, int N, int K, int warmup, int iters, int outer, size_t rotate_bytes, double* min_s,
+HELIX_API int helix_bench(int M, int N, int K, int warmup, int iters, int outer, size_t rotate_bytes, double* min_s,
                 double* avg_s, double* max_s);
 
 /* Same for the convolution entry point.
  * Replaces: `im2col ...` timing main (src_template/Ampere_FP16/im2col.cu:118-196) plus the GEMM run. */
-int helix_bench_conv(int batch, int IC, int H, int W, int OC, int kH, int kW, int stride, int pad, int warmup,
+HELIX_API int helix_bench_conv(int batch, int IC, int H, int W, int OC, int kH, int kW, int stride, int pad, int warmup,
                      int iters, int outer, double* min_s, double* avg_s, double* max_s);
 
 #ifdef __cplusplus

@@ -357,7 +357,7 @@ def test_cli_unsupported_combination_message():
 # ---- C ABI ------------------------------------------------------------------------------------------------------
 def _declared_symbols():
     text = open(os.path.join(ROOT, "include", "helix_abi.h")).read()
-    return sorted(set(re.findall(r"^(?:int|size_t)\s+(helix_\w+)\s*\(", text, flags=re.M)))
+    return sorted(set(re.findall(r"^HELIX_API\s+(?:int|size_t)\s+(helix_\w+)\s*\(", text, flags=re.M)))
 
 
 def test_header_matches_binding():
@@ -381,6 +381,23 @@ def test_every_built_library_exports_the_whole_abi():
         info = hip_ctypes.HelixLib(path).info()
         assert info["arch"] == "gfx950" and info["family"] in ("gemm_f16", "gemv_f16", "sgemm_f32", "gemv_f32", "rocblas_f16", "rocblas_f32",
                                                            "miopen")
+
+
+def test_libraries_export_only_the_abi():
+    """Every library carries its own copy of the tile code (same C++ names, different constants): nothing but the
+    helix_* entry points may be visible to the dynamic linker, or a process holding two configurations could bind
+    one library's entry points to the other's tile code."""
+    libs = _built_libraries()
+    if not libs:
+        pytest.skip("kernel libraries are not built (run __graft_entry__.build())")
+    want = set(_declared_symbols())
+    for path in libs:
+        out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+        names = {line.split()[-1] for line in out.splitlines() if line.strip()}
+        # __hip_cuid_<hash>: the compilation-unit id hipcc emits; _ZSt19piecewise_construct: an empty libstdc++ tag object
+        extra = {n for n in names - want if not n.startswith("__hip_cuid_") and n != "_ZSt19piecewise_construct"}
+        assert not extra, (path, sorted(extra)[:5])
+        assert want <= names, path
 
 
 def test_all_expected_libraries_are_built():
