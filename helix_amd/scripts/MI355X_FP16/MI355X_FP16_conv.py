@@ -12,7 +12,7 @@ import math
 import os
 
 from utils.helix_runtime import load
-from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library
+from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, is_dtl_key
 from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost
 
 root_path = os.getcwd()
@@ -49,12 +49,12 @@ def gather_channels(input_channel):
 
 
 def cost_model(prof_dict, M, N, K, IC=None):
-    """GEMM cost model restricted to the MFMA configurations (the GEMV kernels have no conv path), with the
+    """GEMM cost model restricted to the MFMA configurations with a conv entry (gemm.hip's), with the
     gather terms above; IC is the channel count the kernel walks (gather_channels)."""
     min_cost = float("inf")
     best_config = (1, 1, 1, 1, 1, 0, 32)
     for k, v in prof_dict.items():
-        if k[0] == 0:
+        if k[0] == 0 or is_dtl_key(k):      # neither the GEMV nor the direct-to-LDS libraries have a conv entry
             continue
         cost = conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC)
         if min_cost > cost:

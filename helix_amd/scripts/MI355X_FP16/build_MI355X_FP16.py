@@ -11,6 +11,10 @@ names modulo the backend tag.  Differences that follow from the target:
     pipeline holds the K tile being multiplied in LDS and one more on its way through registers: 2 is the
     only depth the gfx950 template implements), and BLOCK_K is a template parameter too (it is fixed to 32
     in the reference, gemm.cu:77);
+  * the deeper pipelines of the reference (K_STAGE 3 .. 5 are rings of cp.async stages, gemm.cu:156-198) are the
+    direct-to-LDS family, src_template/MI355X_FP16/gemm_dtl.hip: eight-wave tiles whose K tiles go from global
+    memory straight into a ring of K_STAGES LDS stages of BLOCK_K = 32 or 64 columns.  Its prof-dict keys carry a
+    trailing eighth field 1 (DIRECT_TO_LDS); keys of the other families keep seven fields;
   * compiles run in parallel worker threads instead of one os.system at a time.
 """
 import os
@@ -30,6 +34,10 @@ WAVE_TILE_LIST = [32, 64, 128]              # wave-tile rows (the epilogue pairs
 WAVE_COLS_LIST = [32, 48, 64, 96, 128]
 BLOCK_SCALE_LIST = [1, 2, 4]
 BLOCK_K_LIST = [64, 128]
+# direct-to-LDS family: (BLOCK_K, K_STAGES) points.  Three or four 32-column stages keep two or three K tiles in
+# flight; 64-column stages fit the 256 x 256 tile twice only
+DTL_BK_STAGES_LIST = [(32, 3), (32, 4), (64, 2), (64, 3)]
+DTL_BLOCK_SCALES = [(2, 4), (4, 2)]     # eight waves: two per SIMD
 LDS_LIMIT = 160 * 1024
 VGPR_FILE = 512             # registers per lane of one SIMD (arch + accumulation), shared by its resident waves
 
@@ -95,6 +103,53 @@ def iter_configs():
                             yield (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K)
 
 
+def is_valid_dtl_config(block_rows_scale, block_cols_scale, block_rows, block_cols, wave_rows, wave_cols, block_k,
+                        k_stages):
+    """Validity of a point of the direct-to-LDS family (the static_asserts of gemm_dtl.hip)."""
+    # the reference's tile rules (build_Ampere_FP16.py:30-39)
+    if block_rows > 256 or block_cols > 256:
+        return False
+    if wave_cols == wave_rows * 8 or wave_rows == wave_cols * 8:
+        return False
+    if block_cols == block_rows * 16 or block_rows == block_cols * 16:
+        return False
+    if block_rows_scale * block_cols_scale != 8:
+        return False
+    # each of the four copying waves fills whole 1 KiB pieces of a stage: 16 / 8 / 4 matrix rows per instruction
+    rows_per_copy = {32: 16, 64: 8, 128: 4}[block_k]
+    if (block_rows // 4) % rows_per_copy or (block_cols // 4) % rows_per_copy:
+        return False
+    copies = (block_rows // 4 + block_cols // 4) // rows_per_copy
+    if (k_stages - 2) * copies > 63:
+        return False
+    strips = 8 * 32 * (wave_cols * 2 + 16)
+    if max(k_stages * (block_rows + block_cols) * block_k * 2, strips) + 64 > LDS_LIMIT:
+        return False
+    # accumulators plus a whole K tile of fragments in the 256 registers of a wave
+    tm, tn = wave_rows // 16, wave_cols // 16
+    if (block_k // 32) * (tm + tn) * 4 + tm * tn * 4 > 236:
+        return False
+    return True
+
+
+def iter_dtl_configs():
+    """Yields (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) of the direct-to-LDS family."""
+    for (BLOCK_K, K_STAGES) in DTL_BK_STAGES_LIST:
+        for WAVE_ROWS in WAVE_TILE_LIST:
+            for WAVE_COLS in WAVE_COLS_LIST:
+                for (BLOCK_ROWS_SCALE, BLOCK_COLS_SCALE) in DTL_BLOCK_SCALES:
+                    BLOCK_ROWS = BLOCK_ROWS_SCALE * WAVE_ROWS
+                    BLOCK_COLS = BLOCK_COLS_SCALE * WAVE_COLS
+                    if is_valid_dtl_config(BLOCK_ROWS_SCALE, BLOCK_COLS_SCALE, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS,
+                                           WAVE_COLS, BLOCK_K, K_STAGES):
+                        yield (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K)
+
+
+def is_dtl_key(key):
+    """Keys of the direct-to-LDS family carry a trailing eighth field 1."""
+    return len(key) > 7 and key[7] == 1
+
+
 def kernel_library(kernel_name, k_stages=None, block_rows=None, block_cols=None, wave_rows=None, wave_cols=None,
                    block_k=None):
     """Path of the shared library of one configuration (same naming scheme as the reference's
@@ -112,6 +167,8 @@ def library_for_key(key):
     (scripts/Ampere_FP16/Ampere_FP16_gemm.py:435)."""
     if key[0] == 0:
         return kernel_library("gemv" if key[5] == 0 else "gemv_splitK")
+    if is_dtl_key(key):
+        return kernel_library("gemm_dtl", key[0], key[1], key[2], key[3], key[4], key[6])
     return kernel_library("gemm" if key[5] == 0 else "gemm_splitK", key[0], key[1], key[2], key[3], key[4], key[6])
 
 
@@ -148,6 +205,8 @@ def build_jobs():
         jobs.append(compile_job("gemm", *cfg))
         if cfg[0] in SPLITK_STAGES_LIST:
             jobs.append(compile_job("gemm_splitK", *cfg))
+    for cfg in iter_dtl_configs():
+        jobs.append(compile_job("gemm_dtl", *cfg))
     jobs.append(compile_job("gemv"))
     jobs.append(compile_job("gemv_splitK"))
     jobs.append(rocblas_job())

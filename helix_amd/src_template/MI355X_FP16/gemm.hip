@@ -9,7 +9,8 @@
 // operand layout (B stored N x K) follows gemm.cu:144,597-601; unlike the reference's
 // `mma...f16.f16.f16.f16` (gemm.cu:54-57) accumulation is FP32.
 //
-// Compile-time parameters (set with -D by the build script, one shared library per combination):
+// Compile-time parameters (set with -D by the build script, one shared library per combination; gemm_tile.h holds
+// their defaults and the parts shared with the direct-to-LDS template gemm_dtl.hip):
 //   BLOCK_ROWS x BLOCK_COLS   workgroup tile of C           (reference BLOCK_ROWS / BLOCK_COLS)
 //   WAVE_ROWS  x WAVE_COLS    tile of C owned by one wave64 (reference WARP_ROWS / WARP_COLS)
 //   BLOCK_K                   K extent of one LDS stage (64 or 128)
@@ -35,102 +36,30 @@
 //   * workgroup id -> tile: ids are dealt round-robin to the 8 XCDs by the hardware, so id is first
 //     remapped to (xcd, slot) -> xcd * ids_per_xcd + slot, then walked in column-major groups of
 //     GROUP_ROWS tile rows; each XCD's L2 then sees a compact patch of tiles sharing A and B panels.
-#include <hip/hip_runtime.h>
-#include <stdint.h>
-
-#include <type_traits>
-
-#include "helix_abi.h"
+#include "gemm_tile.h"
 #include "helix_im2col.h"
-#include "helix_fastdiv.h"
-
-#ifndef BLOCK_ROWS
-#define BLOCK_ROWS 256
-#endif
-#ifndef BLOCK_COLS
-#define BLOCK_COLS 256
-#endif
-#ifndef WAVE_ROWS
-#define WAVE_ROWS 128
-#endif
-#ifndef WAVE_COLS
-#define WAVE_COLS 128
-#endif
-#ifndef BLOCK_K
-#define BLOCK_K 64
-#endif
-#ifndef K_STAGES
-#define K_STAGES 2
-#endif
-#ifndef SPLIT_K
-#define SPLIT_K 1
-#endif
-#ifndef GROUP_ROWS
-#define GROUP_ROWS 4
-#endif
 
 namespace {
 
-typedef _Float16 half_t;
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half4 __attribute__((ext_vector_type(4)));
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-typedef int intx4 __attribute__((ext_vector_type(4)));
-typedef int intx2 __attribute__((ext_vector_type(2)));
-
-constexpr int BM = BLOCK_ROWS, BN = BLOCK_COLS, WM = WAVE_ROWS, WN = WAVE_COLS, BK = BLOCK_K;
-constexpr int STAGES = K_STAGES, SPLITK = SPLIT_K;
-constexpr int WAVES_M = BM / WM, WAVES_N = BN / WN, NWAVES = WAVES_M * WAVES_N, NTHREADS = 64 * NWAVES;
-constexpr int TM = WM / 16, TN = WN / 16;      // MFMA tiles per wave
 constexpr int KCH = BK / 8;                    // 16-byte chunks per LDS row
 constexpr int ROW_BYTES = BK * 2;
 constexpr int RP = ROW_BYTES >= 256 ? 1 : 256 / ROW_BYTES;  // rows per 256 bytes of LDS
 constexpr int A_ITERS = BM * KCH / NTHREADS, B_ITERS = BN * KCH / NTHREADS;
 constexpr int ROWS_PER_ITER = NTHREADS / KCH;
-constexpr int A_STAGE_BYTES = BM * ROW_BYTES, B_STAGE_BYTES = BN * ROW_BYTES;
-constexpr int STAGE_BYTES = A_STAGE_BYTES + B_STAGE_BYTES;
 constexpr int RING_BYTES = 2 * STAGE_BYTES;
-// epilogue staging: one 32 x WAVE_COLS strip of halves per wave, rows padded by 16 bytes
-constexpr int STRIP_LD = WN * 2 + 16;
-constexpr int STRIP_BYTES = 32 * STRIP_LD;
 constexpr int LDS_BYTES = RING_BYTES > NWAVES * STRIP_BYTES ? RING_BYTES : NWAVES * STRIP_BYTES;
 
-static_assert(BM % WM == 0 && BN % WN == 0, "block tile must be a multiple of the wave tile");
-static_assert(WM % 32 == 0 && WN % 16 == 0, "wave tile: rows in multiples of 32 (the epilogue pairs 16-row tiles), columns of 16");
 static_assert(BK == 64 || BK == 128, "BLOCK_K holds an even number of 32-wide MFMA k-steps: 64 or 128");
-static_assert(NTHREADS <= 1024 && NTHREADS % KCH == 0, "bad thread count");
+static_assert(NTHREADS % KCH == 0, "bad thread count");
 static_assert((BM * KCH) % NTHREADS == 0 && (BN * KCH) % NTHREADS == 0, "tile copy must divide evenly");
 static_assert(STAGES == 2, "K_STAGES: one K tile staged in registers behind the one in LDS");
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
-static_assert(SPLITK >= 1 && SPLITK <= 8, "SPLIT_K out of range");
-
-using helix_fastdiv::FastDiv;   // division by a run-time constant as multiply and shift
-
-struct ConvGeom {
-    int H, W, IC, OH, OW, kW, stride, pad, M;  // M = batch*OH*OW
-    FastDiv by_OW, by_OH, by_IC, by_kW;
-};
-
-struct Params {
-    const half_t* A;   // GEMM: M x K (lda).  CONV: x, NHWC
-    const half_t* B;   // N x K (ldb).        CONV: w, [OC][kH][kW][IC]
-    half_t* C;         // M x N (ldc)
-    float* ws;         // SPLIT_K > 1: [splits][M][N] FP32 partial sums
-    int splits;        // K partitions of this launch (1 when SPLIT_K == 1)
-    int M, N, K, lda, ldb, ldc;
-    int tiles_m, tiles_n;
-    unsigned a_bytes;  // CONV: size of x in bytes (bounds for the gather)
-    ConvGeom g;
-};
 
 __device__ __forceinline__ int swz_key(int row) { return (row / RP) & (KCH - 1); }
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
-
-constexpr int OOB_OFFSET = 0x7fffffff;  // byte offset beyond any buffer: the load returns zeros
-constexpr int KSTEPS = BK / 32;         // MFMA k-steps per K tile (2 or 4)
 
 __device__ __forceinline__ intx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) {
     return __builtin_bit_cast(intx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
@@ -205,7 +134,7 @@ constexpr Schedule make_schedule() {
     return sc;
 }
 
-// The tile parameters appear as (otherwise unused) template arguments so that every configuration's
+
 // kernel has its own symbol name and a profiler lists configurations separately.
 // MODE: 0 = GEMM; 1 = convolution, general gather (tap and channel of every 16-byte chunk computed per K
 // tile); 2 = convolution with IC a multiple of BLOCK_K and at most 32 filter taps: a K tile then lies inside
@@ -221,33 +150,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: lives in a scalar register
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
 
-    // ---- workgroup id -> (tile_m, tile_n), XCD-aware ------------------------------------------
-    const int ntiles = p.tiles_m * p.tiles_n;
-    int pid = blockIdx.x;
-    {
-        const int per = ntiles / 8, rem = ntiles % 8;
-        const int xcd = pid % 8, slot = pid / 8;
-        pid = xcd * per + (xcd < rem ? xcd : rem) + slot;
-    }
-    const int group_tiles = GROUP_ROWS * p.tiles_n;
-    const int grp = pid / group_tiles;
-    const int first_m = grp * GROUP_ROWS;
-    const int gsize = (p.tiles_m - first_m) < GROUP_ROWS ? (p.tiles_m - first_m) : GROUP_ROWS;
-    const int in_grp = pid % group_tiles;
-    const int tile_m = first_m + in_grp % gsize;
-    const int tile_n = in_grp / gsize;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-
-    // ---- K range of this workgroup (split-K partitions are multiples of BLOCK_K) -----------------
-    int k_begin = 0, k_end = p.K;
-    if (SPLITK > 1) {
-        const int ktiles = (p.K + BK - 1) / BK;
-        const int per = (ktiles + p.splits - 1) / p.splits;
-        k_begin = (int)blockIdx.y * per * BK;
-        k_end = k_begin + per * BK;
-        if (k_end > p.K) k_end = p.K;
-        if (k_begin > p.K) k_begin = p.K;
-    }
+    const TileRange tr = tile_range_of_workgroup(p);
+    const int m0 = tr.m0, n0 = tr.n0, k_begin = tr.k_begin, k_end = tr.k_end;
 
     // ---- per-thread copy geometry ---------------------------------------------------------------
     // Copy slot c = tid + i*NTHREADS of a tile lands at LDS byte c*16 (so one wave-wide copy instruction
@@ -537,97 +441,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         stage ^= 1;
     }
 
-    // ---- epilogue ---------------------------------------------------------------------------------
-    // The MFMAs were issued with the B fragment as the first operand, so accumulator tile (i, j) holds the
-    // transposed 16x16 block: lane l owns tile row m = l % 16 and the four consecutive tile columns
-    // n = 4*(l/16) + {0,1,2,3}.
-    const int m_l = lane & 15, n_l = (lane >> 4) * 4;
-    if (SPLITK > 1) {
-        // FP32 partial sums: four consecutive columns per lane, one 16-byte store where that is aligned
-        const bool vec_ok = (p.N % 4 == 0);
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int row = m0 + wave_m * WM + i * 16 + m_l;
-#pragma unroll
-            for (int j = 0; j < TN; j++) {
-                const int col = n0 + wave_n * WN + j * 16 + n_l;
-                if (row < p.M) {
-                    float* dst = p.ws + ((size_t)blockIdx.y * p.M + row) * p.N + col;
-                    if (vec_ok && col + 4 <= p.N) {
-                        *(floatx4*)dst = acc[i][j];
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            if (col + e < p.N) dst[e] = acc[i][j][e];
-                    }
-                }
-            }
-        }
-    } else {
-        // FP16 result through LDS: each wave rounds a 32 x WAVE_COLS strip into its private LDS region
-        // (8-byte writes), reads it back row-contiguous and stores 16 bytes per lane, so a store
-        // instruction covers whole 2*WAVE_COLS-byte row segments.
-        __syncthreads();   // every wave is done reading the ring; the strips reuse its memory
-        unsigned char* strip = smem + wave * STRIP_BYTES;
-        // widest store the row stride and base address allow: 8, 4, 2 or 1 halves at a time
-        const int valign = (int)(((uintptr_t)p.C >> 1) | (unsigned)p.ldc) & 7;
-        const int vec = (valign == 0) ? 8 : (valign & 3) == 0 ? 4 : (valign & 1) == 0 ? 2 : 1;
-        constexpr int CPR = WN / 8;                    // 16-byte chunks per strip row
-#pragma unroll
-        for (int ii = 0; ii < TM / 2; ii++) {
-#pragma unroll
-            for (int hh = 0; hh < 2; hh++) {
-#pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const floatx4 a = acc[ii * 2 + hh][j];
-                    half4 h = {(half_t)a[0], (half_t)a[1], (half_t)a[2], (half_t)a[3]};
-                    *(half4*)(strip + (hh * 16 + m_l) * STRIP_LD + (j * 16 + n_l) * 2) = h;
-                }
-            }
-            __builtin_amdgcn_wave_barrier();   // same-wave LDS traffic stays in program order
-#pragma unroll
-            for (int t = 0; t < (32 * CPR) / 64; t++) {
-                const int idx = t * 64 + lane;
-                const int r = idx / CPR, ch = idx % CPR;
-                const intx4 v = *(const intx4*)(strip + r * STRIP_LD + ch * 16);
-                const int row = m0 + wave_m * WM + ii * 32 + r;
-                const int col = n0 + wave_n * WN + ch * 8;
-                if (row < p.M && col < p.N) {
-                    half_t* dst = p.C + (size_t)row * p.ldc + col;
-                    if (vec == 8 && col + 8 <= p.N) {
-                        *(intx4*)dst = v;
-                    } else if (vec == 4 && col + 8 <= p.N) {
-                        ((intx2*)dst)[0] = intx2{v[0], v[1]};
-                        ((intx2*)dst)[1] = intx2{v[2], v[3]};
-                    } else if (vec == 2 && col + 8 <= p.N) {
-#pragma unroll
-                        for (int e = 0; e < 4; e++) ((int*)dst)[e] = v[e];
-                    } else {
-                        const half8 hv = __builtin_bit_cast(half8, v);
-#pragma unroll
-                        for (int e = 0; e < 8; e++)
-                            if (col + e < p.N) dst[e] = hv[e];
-                    }
-                }
-            }
-            __builtin_amdgcn_wave_barrier();
-        }
-    }
+    store_tile(acc, p, m0, n0, wave, wave_m, wave_n, lane, smem);
 }
-
-// Sums the SPLIT_K FP32 partials in a fixed order and rounds once to FP16 (deterministic, unlike
-// the reference's half2 atomics, src_template/Ampere_FP16/gemm_splitK.cu:495-506).
-__global__ void helix_splitk_reduce_kernel(const float* ws, half_t* C, int M, int N, int ldc, int splits) {
-    const size_t total = (size_t)M * N;
-    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (size_t)gridDim.x * blockDim.x) {
-        float s = 0.f;
-        for (int k = 0; k < splits; k++) s += ws[(size_t)k * total + idx];
-        const size_t row = idx / N, col = idx % N;
-        C[row * ldc + col] = (half_t)s;
-    }
-}
-
 }  // namespace
 
 // -------------------------------------------------------------------------------------------------
@@ -637,8 +452,6 @@ __global__ void helix_splitk_reduce_kernel(const float* ws, half_t* C, int M, in
 
 namespace tpl {
 
-constexpr int kElemBytes = 2;
-
 inline const char* info_json() {
     static char buf[1024];
     static bool done = false;
@@ -646,37 +459,14 @@ inline const char* info_json() {
         snprintf(buf, sizeof(buf),
                  "{\"family\": \"gemm_f16\", \"arch\": \"gfx950\", \"mfma\": \"v_mfma_f32_16x16x32_f16\", "
                  "\"k_stages\": %d, \"block_rows\": %d, \"block_cols\": %d, \"wave_rows\": %d, \"wave_cols\": %d, "
-                 "\"block_k\": %d, \"split_k\": %d, \"threads\": %d, \"lds_bytes\": %d, "
+                 "\"block_k\": %d, \"split_k\": %d, \"direct_to_lds\": %d, \"threads\": %d, \"lds_bytes\": %d, "
                  "\"layout_a\": \"M x K row-major f16\", \"layout_b\": \"N x K row-major f16\", "
                  "\"layout_c\": \"M x N row-major f16\", \"accumulate\": \"f32\", "
                  "\"k_multiple\": 8, \"ld_multiple\": 8, \"conv\": \"NHWC x [OC][kH][kW][IC]; implicit GEMM when IC %% 8 == 0, else column buffer in the workspace\"}",
-                 STAGES, BM, BN, WM, WN, BK, SPLITK, NTHREADS, LDS_BYTES);
+                 STAGES, BM, BN, WM, WN, BK, SPLITK, 0, NTHREADS, LDS_BYTES);
         done = true;
     }
     return buf;
-}
-
-// K partitions for an M x N x K problem: enough to hand every one of the 256 compute units a workgroup,
-// at least 2 (the reference's split-K is always 2-way, gemm_splitK.cu:124-129), at most SPLIT_K, and
-// never so many that a partition has fewer than two K tiles.
-inline int split_factor(long long M, long long N, long long K) {
-    if (SPLITK <= 1) return 1;
-    const long long tiles = ((M + BM - 1) / BM) * ((N + BN - 1) / BN);
-    const long long ktiles = (K + BK - 1) / BK;
-    long long s = 256 / (tiles > 0 ? tiles : 1);
-    if (s > SPLITK) s = SPLITK;
-    if (s > ktiles / 2) s = ktiles / 2;
-    if (s < 2) s = 2;
-    return (int)s;
-}
-
-inline size_t workspace_bytes(int M, int N, int K) {
-    return SPLITK > 1 ? (size_t)split_factor(M, N, K) * (size_t)M * (size_t)N * sizeof(float) : 0;
-}
-
-inline void bench_layout(int M, int N, int K, size_t* ae, size_t* be, size_t* ce, int* lda, int* ldb, int* ldc) {
-    *ae = (size_t)M * K; *be = (size_t)N * K; *ce = (size_t)M * N;
-    *lda = K; *ldb = K; *ldc = N;
 }
 
 template <int MODE>

@@ -22,6 +22,7 @@ import torch
 from oracle import oracle as O
 from utils import seeded_inputs
 from utils.helix_runtime import load
+from utils.hip_ctypes import HELIX_ERR_UNSUPPORTED
 from utils import get_benchmark_shape_list as shapes
 from MI355X_FP16 import build_MI355X_FP16 as b16
 from MI355X_FP16 import profile_MI355X_FP16 as p16
@@ -92,6 +93,11 @@ def test_every_fp16_library_integer_exact(keys):
         for (A, B, exact) in gemms:
             got = run_gemm_f16(lib, A, B)
             assert np.array_equal(got.astype(np.int64), exact), (key, A.shape, B.shape)
+        if b16.is_dtl_key(key):      # the direct-to-LDS family has no convolution entry
+            t = torch.zeros(4096, dtype=torch.float16, device="cuda:0")
+            assert lib.conv2d(t.data_ptr(), t.data_ptr(), t.data_ptr(), 1, 4, 4, 8, 8, 1, 1, 1, 0, check=False) == \
+                HELIX_ERR_UNSUPPORTED
+            continue
         for (x, w, stride, pad, exact) in convs:
             got = run_conv(lib, x, w, stride, pad, torch.float16)
             assert np.array_equal(got.astype(np.float32), exact), (key, x.shape, w.shape)

@@ -25,6 +25,7 @@ from MI355X_FP32 import MI355X_FP32_conv as c32
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 N_FP16_CONFIGS = 159   # points of the FP16 template space (tile x wave tile x BLOCK_K) that fit LDS and registers
 N_FP16_SPLITK = 159    # every point also has a split-K variant
+N_FP16_DTL = 68        # points of the direct-to-LDS family: eight-wave tiles x (BLOCK_K, K_STAGES) in {32: 3, 4; 64: 2, 3}
 
 
 # ---- enumeration ----------------------------------------------------------------------------------
@@ -54,9 +55,33 @@ def test_fp16_template_space():
         assert b16.vgpr_estimate(br, bc, wr, wc, bk) <= 512 // ((threads // 64 + 3) // 4)
     assert (2, 256, 256, 128, 128, 64) in cfgs
     keys = p16.all_keys()
-    assert len(keys) == N_FP16_CONFIGS + N_FP16_SPLITK + 6
-    assert all(len(k) == 7 for k in keys)
+    assert len(keys) == N_FP16_CONFIGS + N_FP16_SPLITK + N_FP16_DTL + 6
+    # seven fields; the direct-to-LDS family carries a trailing eighth field 1
+    assert all(len(k) == (8 if b16.is_dtl_key(k) else 7) for k in keys)
+    assert sum(1 for k in keys if b16.is_dtl_key(k)) == N_FP16_DTL
     assert sum(1 for k in keys if k[0] == 0) == 6   # GEMV rows are tagged by a zero first field
+
+
+def test_fp16_direct_to_lds_space():
+    """The K_STAGES x DIRECT_TO_LDS axes: eight waves per workgroup, a ring of 2 .. 4 stages of 32 or 64 columns
+    within the 160 KiB of LDS, accumulators plus one K tile of fragments within 256 registers."""
+    cfgs = list(b16.iter_dtl_configs())
+    assert len(cfgs) == N_FP16_DTL and len(set(cfgs)) == N_FP16_DTL
+    for (st, br, bc, wr, wc, bk) in cfgs:
+        assert (br // wr) * (bc // wc) == 8 and br <= 256 and bc <= 256
+        assert (bk, st) in b16.DTL_BK_STAGES_LIST and st * (br + bc) * bk * 2 + 64 <= 160 * 1024
+        rows_per_copy = {32: 16, 64: 8}[bk]     # matrix rows one 1 KiB copy instruction fills
+        assert (br // 4) % rows_per_copy == 0 and (bc // 4) % rows_per_copy == 0
+        assert (bk // 32) * (wr // 16 + wc // 16) * 4 + (wr // 16) * (wc // 16) * 4 <= 236
+    assert (4, 256, 256, 128, 64, 32) in cfgs and (2, 256, 256, 128, 64, 64) in cfgs
+    assert (3, 256, 256, 128, 64, 64) not in cfgs       # three 64-column stages of a 256 x 256 tile exceed the LDS
+    assert b16.library_for_key((4, 256, 256, 128, 64, 0, 32, 1)).endswith("build/bin_fp16/libgemm_dtl_4_256_256_128_64_32.so")
+    src, out, defines = b16.compile_job("gemm_dtl", 4, 256, 256, 128, 64, 32)
+    assert src.endswith("src_template/MI355X_FP16/gemm_dtl.hip") and defines["K_STAGES"] == 4 and defines["BLOCK_K"] == 32
+    # no convolution entry: the conv cost model never picks the family
+    d = {(4, 256, 256, 128, 64, 0, 32, 1): 1e-9, (2, 128, 128, 64, 64, 0, 64): 1.0}
+    assert c16.cost_model(d, 4096, 256, 576, 64) == (2, 128, 128, 64, 64, 0, 64)
+    assert g16.cost_model(d, 4096, 4096, 4096) == (4, 256, 256, 128, 64, 0, 32, 1)
 
 
 def test_fp16_library_names():
