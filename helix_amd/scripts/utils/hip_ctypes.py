@@ -13,12 +13,14 @@ HELIX_OK = 0
 HELIX_ERR_INVALID_VALUE = 1
 HELIX_ERR_UNSUPPORTED = 801
 HELIX_ERR_WORKSPACE = 2001
+STATIC_SCRATCH_BYTES = 16 << 20      # HELIX_STATIC_SCRATCH_BYTES of include/helix_abi.h
 
 ABI_SYMBOLS = (
     "helix_info",
     "helix_workspace_bytes",
     "helix_conv_workspace_bytes",
     "helix_gemm",
+    "helix_gemm_static_scratch",
     "helix_conv2d",
     "helix_gemm_timed",
     "helix_conv2d_timed",
@@ -53,6 +55,8 @@ class HelixLib:
         L.helix_conv_workspace_bytes.restype = _sz
         L.helix_gemm.argtypes = [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]
         L.helix_gemm.restype = _i
+        L.helix_gemm_static_scratch.argtypes = [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]
+        L.helix_gemm_static_scratch.restype = _i
         L.helix_conv2d.argtypes = [_vp, _vp, _vp] + [_i] * 9 + [_vp, _sz, _vp]
         L.helix_conv2d.restype = _i
         L.helix_gemm_timed.argtypes = [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _i, _i, _dp]
@@ -86,6 +90,14 @@ class HelixLib:
         rc = self._lib.helix_gemm(A, B, C, M, N, K, lda, ldb, ldc, ws or None, ws_bytes, stream or None)
         if check and rc != 0:
             raise HelixError("helix_gemm", rc)
+        return rc
+
+    def gemm_static_scratch(self, A, B, C, M, N, K, lda, ldb, ldc, stream=0, check=True):
+        """helix_gemm without a workspace argument and without any allocation: K-partition partial sums go to
+        the library's own fixed device array (STATIC_SCRATCH_BYTES); larger needs return HELIX_ERR_WORKSPACE."""
+        rc = self._lib.helix_gemm_static_scratch(A, B, C, M, N, K, lda, ldb, ldc, stream or None)
+        if check and rc != 0:
+            raise HelixError("helix_gemm_static_scratch", rc)
         return rc
 
     def conv2d(self, x, w, y, batch, H, W, IC, OC, kH, kW, stride, pad, ws=0, ws_bytes=0, stream=0, check=True):

@@ -55,4 +55,5 @@ inline int conv2d(const void*, const void*, void*, int, int, int, int, int, int,
 
 }  // namespace tpl
 
+#define HELIX_NO_STATIC_SCRATCH   // the vendor library owns its workspace
 #include "helix_host.h"

@@ -155,6 +155,59 @@ int helix_conv2d(const void* x, const void* w, void* y, int batch, int H, int W,
                        (hipStream_t)stream);
 }
 
+#ifndef HELIX_NO_STATIC_SCRATCH
+}  // extern "C"
+
+// Scratch memory of helix_gemm_static_scratch: the K-partition partial sums live in this array instead of in
+// a caller-provided workspace.  Every GPU the library runs on holds its own copy of the array, at its own
+// address, until the process ends.  In host code the name is only a handle for HIP_SYMBOL(); the memory is
+// reached through the per-device pointer below.
+static __device__ __align__(256) unsigned char scratch[HELIX_STATIC_SCRATCH_BYTES];
+
+namespace helix_host {
+namespace {
+
+constexpr int kMaxDevices = 64;
+void* scratch_ptr[kMaxDevices];   // device address of `scratch` per device ordinal, filled on first use
+
+// Device address of `scratch` on the current device (looked up once per device, with that device current).
+inline int static_scratch(void** out) {
+    int d = -1;
+    HELIX_HIP_TRY(hipGetDevice(&d));
+    if (d < 0 || d >= kMaxDevices) return HELIX_ERR_INVALID_VALUE;
+    void* p = __atomic_load_n(&scratch_ptr[d], __ATOMIC_ACQUIRE);
+    if (!p) {
+        HELIX_HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return HELIX_ERR_INVALID_VALUE;
+        __atomic_store_n(&scratch_ptr[d], p, __ATOMIC_RELEASE);   // racing first calls store the same address
+    }
+    *out = p;
+    return 0;
+}
+
+}  // namespace
+}  // namespace helix_host
+
+extern "C" {
+
+int helix_gemm_static_scratch(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
+                              void* stream) {
+    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return HELIX_ERR_INVALID_VALUE;
+    const size_t need = tpl::workspace_bytes(M, N, K);
+    if (need > (size_t)HELIX_STATIC_SCRATCH_BYTES) return HELIX_ERR_WORKSPACE;
+    void* ws = nullptr;
+    int rc = helix_host::static_scratch(&ws);
+    if (rc) return rc;
+    // Nothing to clear: a K-partitioned launch writes every partial sum of its M x N x partitions block before
+    // its reduction pass reads that block, and reads nothing else of the array.
+    return tpl::gemm(A, B, C, M, N, K, lda, ldb, ldc, ws, (size_t)HELIX_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
+}
+#else
+int helix_gemm_static_scratch(const void*, const void*, void*, int, int, int, int, int, int, void*) {
+    return HELIX_ERR_UNSUPPORTED;   // vendor comparator: the vendor library manages (and may allocate) its own workspace
+}
+#endif
+
 int helix_gemm_timed(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
                      void* workspace, size_t workspace_bytes, void* stream, int warmup, int iters,
                      double* avg_s) {

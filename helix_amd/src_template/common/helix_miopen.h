@@ -119,4 +119,5 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
 
 }  // namespace tpl
 
+#define HELIX_NO_STATIC_SCRATCH   // the vendor library owns its workspace
 #include "helix_host.h"

@@ -70,6 +70,21 @@ HELIX_API size_t helix_workspace_bytes(int M, int N, int K);
 HELIX_API int helix_gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc,
                void* workspace, size_t workspace_bytes, void* stream);
 
+/* `helix_gemm` for callers that cannot allocate device memory or pass a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the K-partition partial sums go to a
+ * fixed array of HELIX_STATIC_SCRATCH_BYTES inside the library's device image, so the call allocates
+ * nothing and needs no workspace argument.  Same kernels, same results as `helix_gemm` with the workspace
+ * `helix_workspace_bytes` asks for.  A shape that needs more than HELIX_STATIC_SCRATCH_BYTES returns
+ * HELIX_ERR_WORKSPACE and launches nothing; the vendor comparator libraries return HELIX_ERR_UNSUPPORTED.
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (different streams or host
+ * threads) race on it; calls on one stream are ordered and safe.  The array keeps the last call's
+ * contents; nothing needs clearing because a launch writes every partial sum it later reads.  The first
+ * launch of a library on a device loads its code object like any first launch: warm up before capturing.
+ * No counterpart in the reference: it exists for the callers named above, those that cannot allocate. */
+#define HELIX_STATIC_SCRATCH_BYTES (16u << 20)
+HELIX_API int helix_gemm_static_scratch(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb,
+                                        int ldc, void* stream);
+
 /* Bytes of device scratch `helix_conv2d` needs for this problem: the split-K partial sums of the implicit
  * GEMM, plus -- when IC is not a multiple of the 16-byte gather chunk (8 halves / 4 floats) -- the
  * channel-padded copies of activations and weights, or (IC = 1; 2 in FP16) the column buffer and repacked
