@@ -35,6 +35,7 @@ class Backend:
         self.gemm_result = getattr(self.gemm, f"get_{name}_gemm_Helix_result")
         self.gemm_oracle = getattr(self.gemm, f"get_{name}_gemm_Oracle_result")
         self.conv_result = getattr(self.conv, f"get_{name}_conv_Helix_result")
+        self.gemm_vendor = getattr(self.gemm, f"get_{name}_gemm_rocblas_result")
 
     def prof_dict(self):
         if not os.path.exists(prof_dict_path(self.name)):
@@ -48,7 +49,9 @@ class Backend:
         return k[0] if self.fp32 else k[1]
 
 
-def square_rows(be, prof_dict, oracle=False):
+def square_rows(be, prof_dict, oracle=False, vendor=False):
+    """Per size: the cost model's pick (Default); oracle=True adds the exhaustive per-shape search, vendor=True
+    rocBLAS on the same operand layouts."""
     rows = []
     for s in S.BASELINE_SQUARE_SIZES:
         key = be.gemm.cost_model(prof_dict, s, s, s)
@@ -59,6 +62,9 @@ def square_rows(be, prof_dict, oracle=False):
             oms, otf, okey = be.gemm_oracle(prof_dict, s, s, s)
             row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2),
                         "oracle_frac_mfma_peak": round(otf * 1e12 / be.peak, 4)})
+        if vendor:
+            vms, vtf = be.gemm_vendor(s, s, s)
+            row.update({"rocblas_us": round(vms * 1e3, 2), "rocblas_TFLOP/s": round(vtf, 2)})
         rows.append(row)
     return rows
 
@@ -90,6 +96,9 @@ def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
                                                                    rotate_bytes=rotate_bytes)[0]
                 row["tile_GB/s"] = round(nbytes / mn_t / 1e9, 1)
                 row["tile_config"] = list(best_k)
+                # what the search over both families delivers for the shape
+                row["best_GB/s"] = max(row["GB/s"], row["tile_GB/s"])
+                row["best_frac_hbm_peak"] = round(row["best_GB/s"] * 1e9 / R.HBM_BYTES_PER_S, 4)
             rows.append(row)
     return rows
 
@@ -113,21 +122,43 @@ def conv_rows(be, prof_dict, vendor=False):
     return rows
 
 
-def bert_rows(be, prof_dict):
-    """Per distinct GEMM of the encoder, then the whole list (12 layers + the irregular shape) as one row."""
+def bert_rows(be, prof_dict, oracle=False, vendor=False):
+    """Per distinct GEMM of the encoder, then the whole list (12 layers + the irregular shape) as one row: summed
+    latency, as the reference sums per-GEMM costs (benchmark_Ampere_FP16_model_level_LLM.py:16-27).  oracle=True adds
+    the exhaustive per-shape search ("per-shape autotune"), vendor=True rocBLAS."""
     memo, rows = {}, []
-    total_ms, total_flops = 0.0, 0.0
+    totals = {"default": 0.0, "oracle": 0.0, "rocblas": 0.0}
+    total_flops = 0.0
     for (M, N, K) in S.get_baseline_bert_MNKList():
         if (M, N, K) not in memo:
-            memo[(M, N, K)] = be.gemm_result(prof_dict, M, N, K)
-            ms, tflops = memo[(M, N, K)]
-            rows.append({"M": M, "N": N, "K": K, "config": list(be.gemm.cost_model(prof_dict, M, N, K)),
-                         "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
-                         "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)})
-        total_ms += memo[(M, N, K)][0]
+            ms, tflops = be.gemm_result(prof_dict, M, N, K)
+            row = {"M": M, "N": N, "K": K, "config": list(be.gemm.cost_model(prof_dict, M, N, K)),
+                   "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
+                   "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
+            times = {"default": ms}
+            if oracle:
+                oms, otf, okey = be.gemm_oracle(prof_dict, M, N, K)
+                row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2)})
+                times["oracle"] = oms
+            if vendor:
+                vms, vtf = be.gemm_vendor(M, N, K)
+                row.update({"rocblas_us": round(vms * 1e3, 2), "rocblas_TFLOP/s": round(vtf, 2)})
+                times["rocblas"] = vms
+            memo[(M, N, K)] = times
+            rows.append(row)
+        for name, ms in memo[(M, N, K)].items():
+            totals[name] += ms
         total_flops += 2.0 * M * N * K
-    tf = total_flops / (total_ms * 1e-3) / 1e12
-    rows.append({"total_ms": round(total_ms, 4), "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf * 1e12 / be.peak, 4)})
+    tf = total_flops / (totals["default"] * 1e-3) / 1e12
+    total = {"total_ms": round(totals["default"], 4), "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf * 1e12 / be.peak, 4)}
+    if oracle:
+        otf = total_flops / (totals["oracle"] * 1e-3) / 1e12
+        total.update({"oracle_total_ms": round(totals["oracle"], 4), "oracle_TFLOP/s": round(otf, 2),
+                      "oracle_frac_mfma_peak": round(otf * 1e12 / be.peak, 4)})
+    if vendor:
+        total.update({"rocblas_total_ms": round(totals["rocblas"], 4),
+                      "rocblas_TFLOP/s": round(total_flops / (totals["rocblas"] * 1e-3) / 1e12, 2)})
+    rows.append(total)
     return rows
 
 
@@ -140,7 +171,9 @@ def run(backend, configs, oracle=False, tiles=True, vendor=False):
     out = {}
     for name in configs:
         if name == "square":
-            out[name] = square_rows(be, prof_dict, oracle)
+            out[name] = square_rows(be, prof_dict, oracle, vendor)
+        elif name == "bert":
+            out[name] = bert_rows(be, prof_dict, oracle, vendor)
         elif name == "gemv":
             out[name] = gemv_rows(be, prof_dict, tiles=tiles)
         elif name == "conv":
@@ -154,9 +187,9 @@ if __name__ == "__main__":
     parser = argparse.ArgumentParser(description="Benchmark the measured configurations against their rooflines")
     parser.add_argument("-c", "--config", type=str, choices=list(SECTIONS) + ["all"], default="all")
     parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default="MI355X_FP16")
-    parser.add_argument("--oracle", action="store_true", help="also run the exhaustive search on the square shapes")
+    parser.add_argument("--oracle", action="store_true", help="square, bert: also run the exhaustive per-shape search")
     parser.add_argument("--no-tiles", action="store_true", help="gemv: time the GEMV library only")
-    parser.add_argument("--vendor", action="store_true", help="conv: add MIOpen's time per layer")
+    parser.add_argument("--vendor", action="store_true", help="conv: add MIOpen's time per layer; square, bert: add rocBLAS's")
     parser.add_argument("--json", action="store_true", help="one JSON object instead of the table")
     args = parser.parse_args()
 
