@@ -75,7 +75,7 @@ def other_configs():
     be16, d16 = dicts["MI355X_FP16"]
     out["gemv_hbm"] = bc.gemv_rows(be16, d16)
     out["gemm_f16_squares"] = bc.square_rows(be16, d16, oracle=True, vendor=True)
-    out["conv_f16"] = bc.conv_rows(be16, d16, vendor=True)
+    out["conv_f16"] = bc.conv_rows(be16, d16, vendor=True, oracle=True)
     out["bert_f16"] = bc.bert_rows(be16, d16, oracle=True, vendor=True)[-1]
     be32, d32 = dicts["MI355X_FP32"]
     out["sgemm_f32"] = bc.square_rows(be32, d32, oracle=True, vendor=True)

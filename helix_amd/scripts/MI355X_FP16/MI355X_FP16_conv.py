@@ -11,7 +11,7 @@ repack + GEMM), all on one stream and timed as one.
 import math
 import os
 
-from utils.helix_runtime import load
+from utils.helix_runtime import load, kernel_resources
 from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, is_dtl_key
 from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost
 
@@ -48,6 +48,17 @@ def gather_channels(input_channel):
     return padded if 3 * padded <= 8 * input_channel else input_channel
 
 
+def conv_kernel_scratch(k, IC=None):
+    """Scratch bytes per lane (register spills) of the convolution kernel configuration k runs for this channel count,
+    as recorded when the library was built; 0 when the build left no record.  The gather keeps per-copy-slot state
+    in registers beside the accumulators, so the largest tiles fit the GEMM but spill in a convolution mode."""
+    mode = 2 if (IC is not None and IC % k[6] == 0) else 1     # a K tile inside one filter tap, or the general gather
+    for name, res in kernel_resources(library_for_key(k)).items():
+        if f"helix_gemm_f16_kernelILi{mode}E" in name:
+            return res.get("scratch", 0)
+    return 0
+
+
 def cost_model(prof_dict, M, N, K, IC=None):
     """GEMM cost model restricted to the MFMA configurations with a conv entry (gemm.hip's), with the
     gather terms above; IC is the channel count the kernel walks (gather_channels)."""
@@ -55,6 +66,8 @@ def cost_model(prof_dict, M, N, K, IC=None):
     best_config = (1, 1, 1, 1, 1, 0, 32)
     for k, v in prof_dict.items():
         if k[0] == 0 or is_dtl_key(k):      # neither the GEMV nor the direct-to-LDS libraries have a conv entry
+            continue
+        if conv_kernel_scratch(k, IC) > 0:  # a spilling gather is never the fastest one
             continue
         cost = conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC)
         if min_cost > cost:
@@ -77,6 +90,28 @@ def get_MI355X_FP16_conv_Helix_result(prof_dict, batch, input_channel, H, W, out
     tflops = 2 * M * N * K / 1e9 / cost
 
     return cost, tflops
+
+
+def get_MI355X_FP16_conv_Oracle_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
+    """Exhaustive per-layer search: run every configuration that has a conv entry, keep the fastest (the conv
+    counterpart of benchmark_Ampere_FP16_performance_comparison.py:56-69).  Returns (cost_ms, tflops, key)."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    flops = 2.0 * M * output_channel * input_channel * kH * kW
+    min_cost, best = float("inf"), None
+    for k in prof_dict.keys():
+        if k[0] == 0 or is_dtl_key(k):
+            continue
+        try:
+            _, avg, _ = load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride,
+                                                            pad, warmup=2, iters=5)
+        except Exception:
+            continue
+        if avg < min_cost:
+            min_cost, best = avg, k
+    if best is not None:     # the winner once more with the runner's launch counts
+        _, min_cost, _ = load(library_for_key(best)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW,
+                                                                stride, pad, warmup=10, iters=10)
+    return min_cost * 1e3, flops / 1e12 / min_cost, best
 
 
 def get_MI355X_FP16_conv_miopen_result(batch, input_channel, H, W, output_channel, kH, kW, stride, pad):

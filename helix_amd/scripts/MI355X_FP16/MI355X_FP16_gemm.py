@@ -15,6 +15,10 @@ from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K, PROFILE_K_SHORT
 root_path = os.getcwd()
 
 HBM_SUSTAINED_FRACTION = 0.8  # share of the datasheet HBM rate a streaming kernel sustains
+# ... and what the tile kernels sustain when a problem is a pass over a cold operand (measured 5.2 - 5.5 TB/s on
+# 8192 x 28672 weights): their profile point is a hot 16 x 16-tile problem, so this floor is what ranks them against
+# the weight-streaming kernels, whose profile point is cold
+TILE_HBM_SUSTAINED_FRACTION = 0.68
 GEMV_LAUNCH_FLOOR_S = 3.4e-6       # a kernel launch on an idle queue; keeps tiny problems from looking free
 GEMV_MFMA_FLOOR_S = 6.5e-6         # 9 or more activation rows: the K-partitioned MFMA variant plus its reduction
 GEMV_MFMA_MIN_M = 9                # MFMA_MIN_M of src_template/MI355X_FP16/gemv.hip
@@ -64,7 +68,9 @@ def config_cost(k, v, M, N, K, v_short=None):
             return float("inf")
         num_block = math.ceil(small / k[1]) * math.ceil(big / k[2])
         floor = GEMV_LAUNCH_FLOOR_S if small < GEMV_MFMA_MIN_M else GEMV_MFMA_FLOOR_S
-        cost = max(num_block / NUM_CU * v * max(K, 512) / PROFILE_K, floor)
+        # the profiled launch holds one launch's fixed time, which does not scale with the problem
+        stream = max(v - GEMV_LAUNCH_FLOOR_S, 0.0)
+        cost = max(GEMV_LAUNCH_FLOOR_S + num_block / NUM_CU * stream * max(K, 512) / PROFILE_K, floor)
         return cost + (GEMV_SPLITK_EXTRA_S if k[5] == 1 else 0.0)
     splits = split_factor(k, M, N, K)
     num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * splits
@@ -83,7 +89,7 @@ def config_cost(k, v, M, N, K, v_short=None):
     if v_short is not None:
         cost -= ROUND_OVERLAP_S * (w - 1)
     # a tile round cannot beat streaming every operand once from HBM at the sustained rate
-    return max(cost, gemm_bytes(M, N, K, 2) / (HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
+    return max(cost, gemm_bytes(M, N, K, 2) / (TILE_HBM_SUSTAINED_FRACTION * HBM_BYTES_PER_S))
 
 
 def short_value(prof_dict, k):

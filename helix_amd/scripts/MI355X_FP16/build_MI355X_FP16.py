@@ -182,6 +182,11 @@ def compile_job(kernel_name, k_stages=None, block_rows=None, block_cols=None, wa
     elif kernel_name == "gemv_splitK":
         src_name = "gemv"
         defines["SPLIT_K"] = 4
+    elif kernel_name == "gemv_nomfma":
+        # the wave-reduction kernel for every batch up to 16 rows (no MFMA at all): the number the MFMA variant of
+        # 9 .. 16 rows is reported against
+        src_name = "gemv"
+        defines["MFMA_MIN_M"] = 17
     if k_stages is not None:
         defines["K_STAGES"] = k_stages
     if block_rows is not None:
@@ -209,6 +214,7 @@ def build_jobs():
         jobs.append(compile_job("gemm_dtl", *cfg))
     jobs.append(compile_job("gemv"))
     jobs.append(compile_job("gemv_splitK"))
+    jobs.append(compile_job("gemv_nomfma"))
     jobs.append(rocblas_job())
     jobs.append(miopen_job())
     return jobs

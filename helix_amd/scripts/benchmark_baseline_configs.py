@@ -74,6 +74,9 @@ def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
     library, and (tiles=True) the fastest of the 32-row MFMA tile libraries, the other family the cost model
     chooses from for skinny shapes."""
     lib = load(be.build.kernel_library("gemv_fp32" if be.fp32 else "gemv"))
+    # FP16: the same template with the MFMA variant switched off (vector dot products and a wave reduction for
+    # every batch), reported beside the MFMA variant where the two differ (9 or more activation rows)
+    nomfma = None if be.fp32 else load(be.build.kernel_library("gemv_nomfma"))
     tile_keys = [k for k in prof_dict if not be.is_gemv_key(k) and be.block_rows(k) == 32] if tiles else []
     rows = []
     for (K, N) in S.BASELINE_GEMV_KN:
@@ -82,6 +85,9 @@ def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
             nbytes = R.gemm_bytes(M, N, K, be.elem_bytes)
             row = {"M": M, "K": K, "N": N, "us": round(mn * 1e6, 2), "GB/s": round(nbytes / mn / 1e9, 1),
                    "frac_hbm_peak": round(nbytes / mn / R.HBM_BYTES_PER_S, 4)}
+            if nomfma is not None and M >= 9:
+                mn_v = nomfma.bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)[0]
+                row["no_mfma_GB/s"] = round(nbytes / mn_v / 1e9, 1)
             best_t, best_k = float("inf"), None
             for k in tile_keys:
                 try:
@@ -103,9 +109,11 @@ def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
     return rows
 
 
-def conv_rows(be, prof_dict, vendor=False):
-    """vendor=True adds MIOpen's time on the same layer (the comparator library)."""
+def conv_rows(be, prof_dict, vendor=False, oracle=False):
+    """vendor=True adds MIOpen's time on the same layer (the comparator library); oracle=True the exhaustive
+    per-layer search over every configuration with a conv entry (FP16 backend)."""
     miopen = load(be.build.kernel_library("miopen_f32" if be.fp32 else "miopen_f16")) if vendor else None
+    conv_oracle = getattr(be.conv, f"get_{be.name}_conv_Oracle_result", None) if oracle else None
     rows = []
     for shp in S.get_baseline_conv_shape_list():
         b, ic, h, w, oc, kh, kw, st, pd = shp
@@ -117,6 +125,11 @@ def conv_rows(be, prof_dict, vendor=False):
                      "TFLOP/s": round(tflops, 2), "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4),
                      "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / (ms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
+        if conv_oracle is not None:
+            oms, otf, okey = conv_oracle(prof_dict, *shp)
+            rows[-1].update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2),
+                             "oracle_frac_mfma_peak": round(otf * 1e12 / be.peak, 4),
+                             "oracle_frac_hbm_peak": round(nbytes / (oms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
         if miopen is not None:
             rows[-1]["miopen_us"] = round(miopen.bench_conv(*shp, warmup=10, iters=10)[1] * 1e6, 2)
     return rows
@@ -177,7 +190,7 @@ def run(backend, configs, oracle=False, tiles=True, vendor=False):
         elif name == "gemv":
             out[name] = gemv_rows(be, prof_dict, tiles=tiles)
         elif name == "conv":
-            out[name] = conv_rows(be, prof_dict, vendor=vendor)
+            out[name] = conv_rows(be, prof_dict, vendor=vendor, oracle=oracle)
         else:
             out[name] = SECTIONS[name](be, prof_dict)
     return out
@@ -187,7 +200,7 @@ if __name__ == "__main__":
     parser = argparse.ArgumentParser(description="Benchmark the measured configurations against their rooflines")
     parser.add_argument("-c", "--config", type=str, choices=list(SECTIONS) + ["all"], default="all")
     parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default="MI355X_FP16")
-    parser.add_argument("--oracle", action="store_true", help="square, bert: also run the exhaustive per-shape search")
+    parser.add_argument("--oracle", action="store_true", help="square, bert, conv: also run the exhaustive per-shape search")
     parser.add_argument("--no-tiles", action="store_true", help="gemv: time the GEMV library only")
     parser.add_argument("--vendor", action="store_true", help="conv: add MIOpen's time per layer; square, bert: add rocBLAS's")
     parser.add_argument("--json", action="store_true", help="one JSON object instead of the table")

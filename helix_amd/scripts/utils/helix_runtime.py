@@ -5,7 +5,9 @@ scripts/Ampere_FP16/build_Ampere_FP16.py:7-28) and once per measurement (`os.pop
 scripts/Ampere_FP16/profile_Ampere_FP16.py:36-38).  Here a configuration is a shared library that is
 compiled once, loaded once per process and called through ctypes.
 """
+import json
 import os
+import re
 import subprocess
 import time
 from concurrent.futures import ThreadPoolExecutor
@@ -29,8 +31,10 @@ HIPCC = os.environ.get("HIPCC", "hipcc")
 # -packed-fp32-ops is switched off on purpose: the compiler must not form packed FP32 VALU ops here.
 # Hidden visibility + -Bsymbolic: a library exports the helix_* entry points of include/helix_abi.h and nothing
 # else, and its own calls bind inside it, so several configurations can share a process however they are opened.
+# -Rpass-analysis=kernel-resource-usage: hipcc reports registers, scratch and LDS of every kernel on stderr;
+# compile_many keeps the figures in <bin dir>/resource_usage.json (see kernel_resources).
 COMPILE_OPTIONS = ("-O3 -std=c++17 --offload-arch=gfx950 -shared -fPIC -w -fvisibility=hidden -Wl,-Bsymbolic "
-                   "-Xclang -target-feature -Xclang -packed-fp32-ops")
+                   "-Xclang -target-feature -Xclang -packed-fp32-ops -Rpass-analysis=kernel-resource-usage")
 
 
 def bin_dir(precision):
@@ -66,12 +70,38 @@ def compile_library(src, out, defines, link=""):
     return True, proc.stderr
 
 
+def parse_resource_usage(stderr_text):
+    """{kernel function name: {"vgprs": n, "agprs": n, "scratch": bytes per lane, "occupancy": waves per SIMD}} from
+    the -Rpass-analysis=kernel-resource-usage remarks of one hipcc run."""
+    out, cur = {}, None
+    for line in stderr_text.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            cur = out.setdefault(m.group(1), {})
+            continue
+        if cur is None:
+            continue
+        for label, field in (("VGPRs:", "vgprs"), ("AGPRs:", "agprs"), ("ScratchSize [bytes/lane]:", "scratch"),
+                             ("Occupancy [waves/SIMD]:", "occupancy")):
+            m = re.search(r"remark:\s+" + re.escape(label) + r"\s+(\d+)", line)
+            if m:
+                cur[field] = int(m.group(1))
+    return out
+
+
+def resource_usage_path(directory):
+    return os.path.join(directory, "resource_usage.json")
+
+
 def compile_many(jobs, max_workers=None, progress=None):
-    """jobs: iterable of (src, out, defines[, link flags]).  Compiles in parallel; returns list of failed outs."""
+    """jobs: iterable of (src, out, defines[, link flags]).  Compiles in parallel; returns list of failed outs.
+    The per-kernel register / scratch figures hipcc reports are merged into resource_usage.json next to the
+    libraries, keyed by library file name."""
     jobs = list(jobs)
     if max_workers is None:
         max_workers = int(os.environ.get("MAX_JOBS", min(16, os.cpu_count() or 1)))
     failed = []
+    usage = {}
 
     def run(job):
         ok, err = compile_library(*job)
@@ -81,9 +111,39 @@ def compile_many(jobs, max_workers=None, progress=None):
         for job, ok, err in ex.map(run, jobs):
             if not ok:
                 failed.append((job[1], err))
+            else:
+                usage.setdefault(os.path.dirname(job[1]), {})[os.path.basename(job[1])] = parse_resource_usage(err)
             if progress is not None:
                 progress.update(1)
+    for directory, per_lib in usage.items():
+        path = resource_usage_path(directory)
+        merged = {}
+        if os.path.exists(path):
+            try:
+                with open(path) as f:
+                    merged = json.load(f)
+            except ValueError:
+                merged = {}
+        merged.update(per_lib)
+        with open(path, "w") as f:
+            json.dump(merged, f)
     return failed
+
+
+_resource_cache = {}
+
+
+def kernel_resources(library_path):
+    """The kernels of one built library with their registers and scratch bytes, {} when the build left no record."""
+    directory = os.path.dirname(library_path)
+    if directory not in _resource_cache:
+        path = resource_usage_path(directory)
+        try:
+            with open(path) as f:
+                _resource_cache[directory] = json.load(f)
+        except (OSError, ValueError):
+            _resource_cache[directory] = {}
+    return _resource_cache[directory].get(os.path.basename(library_path), {})
 
 
 _lib_cache = {}

@@ -31,17 +31,18 @@
 //     atomics, gemv_splitK.cu:213-217).
 //
 // MFMA variant (M >= MFMA_MIN_M)
-//   * a workgroup walks its K range in chunks of MFMA_KCHUNK columns and stages 16 activation rows of the
-//     chunk in LDS, rows 16 bytes apart from a multiple of 256 so that 16 rows of one column sit in 16
-//     different bank groups;
-//   * a wave owns runs of 16 consecutive weight rows; per 256-wide K step it issues eight 16-byte loads per
-//     lane, straight into registers in the operand layout of the MFMA (lane l: row l % 16, columns 8*(l/16)
-//     .. +7 of a 32-wide block): 512 contiguous bytes per row and step, 64 per row and instruction; the same
-//     columns of activation row l % 16 come from LDS;
-//   * eight MFMAs per step accumulate the 16 x 16 block y[m][n]; steps are double-buffered; buffer bounds
-//     checking zero-fills weight rows beyond N;
-//   * K is partitioned over blockIdx.z only when the weight rows alone give the launch too few waves to cover
-//     the latency of the stream (FP32 workspace + fixed-order reduce).
+//   * a workgroup (four waves, one per compute unit) walks its K range in chunks of 512 columns and stages 16
+//     activation rows of the chunk in LDS, rows 16 bytes apart from a multiple of 256 so that 16 rows of one column
+//     sit in 16 different bank groups;
+//   * a wave owns runs of 16 consecutive weight rows and streams them through a ring in LDS that is private to it:
+//     every copy instruction (buffer_load ... lds) fetches 512 contiguous bytes of each of two rows -- whole-row
+//     spans, the pattern that streams fastest -- and the MFMA operands (lane l: row l % 16, columns 8*(l/16) .. +7 of
+//     a 32-wide block) are read back from LDS.  Loading the operand layout straight into registers (16 rows x 64
+//     bytes per instruction) measured 4.3 TB/s on 8192 x 28672 weights at 16 rows, this variant 5.3;
+//   * eight MFMAs per 256-column step accumulate the 16 x 16 block y[m][n]; copies run three steps ahead; buffer
+//     bounds checking zero-fills weight rows beyond N;
+//   * groups per wave and K ranges (blockIdx.z; FP32 workspace + fixed-order reduce) are chosen per problem so that
+//     rounds of 1024 waves x the stream of one wave is shortest (stream_split).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -86,14 +87,8 @@
 #ifndef MFMA_MIN_M
 #define MFMA_MIN_M 9        // activation rows from which the MFMA variant takes over (measured crossover)
 #endif
-#ifndef MFMA_TARGET_WAVES
-#define MFMA_TARGET_WAVES 8192
-#endif
-#ifndef MFMA_WAVES_PER_BLOCK
-#define MFMA_WAVES_PER_BLOCK 4
-#endif
-#ifndef MFMA_KCHUNK
-#define MFMA_KCHUNK 1024    // columns of the 16 activation rows staged in LDS at a time by the MFMA variant
+#ifndef STREAM_TARGET_WAVES
+#define STREAM_TARGET_WAVES 1024   // 256 compute units x one workgroup of four waves
 #endif
 
 namespace {
@@ -329,110 +324,173 @@ __global__ __launch_bounds__(64 * WAVES) void helix_gemv_f16_kernel(const Params
     }
 }
 
-// ---- MFMA variant -----------------------------------------------------------------------------------------
-constexpr int MSTEP = 256;                      // K extent of one step: eight 16-byte loads per lane, 512 bytes per weight row
-constexpr int MCH = MSTEP / 32;                 // 16-byte chunks per lane and step = MFMAs per step
-constexpr int MFMA_KCHUNK_MAX = MFMA_KCHUNK;     // staged columns: a multiple of MSTEP
-constexpr int MWPB = MFMA_WAVES_PER_BLOCK;
 constexpr int XROW_PAD = 16;                    // bytes between staged rows: 16 rows of one column hit 16 bank groups
+constexpr int MGROUPS = 8;                      // most 16-row groups one wave owns
 
-#ifndef MFMA_LOAD_AUX
-#define MFMA_LOAD_AUX 0   // cache policy bits of the weight loads (non-temporal, 2, measures 5-10 % slower: the two
-                          // halves of a 128-byte line are fetched by consecutive instructions)
+// ---- MFMA variant: weights streamed through LDS -----------------------------------------------------------------
+// Loading the MFMA operand layout straight into registers means 16 rows x 64 bytes per instruction, a pattern that
+// streams at about two thirds of the rate of whole-row spans.  Here every copy instruction fetches 512 contiguous
+// bytes of each of two weight rows straight into LDS (buffer_load ... lds, no registers in between), into a ring of
+// SRING steps of 16 rows x 256 columns that is private to the wave -- no workgroup barrier in the stream -- and the
+// MFMA operands are read from there: lane (r, q) takes 16-byte chunk 4c + q of row r for MFMA c of the step.
+// Chunk ch of row r is stored at chunk position ch ^ r of the row's 512 bytes, so that the 16 rows of one chunk
+// column sit in 16 different bank groups.  Copies run SRING - 1 steps ahead of the MFMAs and keep running across
+// the workgroup's activation staging and from one 16-row group to the next.
+constexpr int SSTEP = 256;                       // columns per step
+#ifndef STREAM_RING
+#define STREAM_RING 4
 #endif
-__device__ __forceinline__ half8 buf_load8(__amdgpu_buffer_rsrc_t r, int voff, int soff) {
-    return __builtin_bit_cast(half8, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, MFMA_LOAD_AUX));
+#ifndef STREAM_XC
+#define STREAM_XC 512
+#endif
+constexpr int SRING = STREAM_RING;               // ring slots per wave
+constexpr int SAHEAD = SRING - 1;                // steps a copy is issued ahead of its use
+constexpr int SSLOT_BYTES = 16 * SSTEP * 2;      // 8 KiB: 16 rows x 512 bytes
+constexpr int SCOPIES = SSLOT_BYTES / 1024;      // copy instructions per step (8): two rows each
+constexpr int SXC = STREAM_XC;                   // activation columns staged at a time
+constexpr int SWPB = 4;                          // waves per workgroup
+constexpr int SXROW = SXC * 2 + XROW_PAD;        // bytes per staged activation row
+constexpr int SX_BYTES = ((16 * SXROW + 1023) / 1024) * 1024;
+constexpr int STREAM_LDS_BYTES = SX_BYTES + SWPB * SRING * SSLOT_BYTES;
+static_assert(STREAM_LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
+static_assert(SAHEAD * SCOPIES <= 63, "copies in flight are counted in a 6-bit counter");
+
+typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
+
+__device__ __forceinline__ intx4 raw_rsrc(const void* base, unsigned bytes) {
+    const unsigned long long a = (unsigned long long)base;
+    intx4 r = {(int)(unsigned)a, (int)((a >> 32) & 0xffffu), (int)bytes, 0x00020000};
+    return r;
 }
 
-constexpr int MGROUPS = 4;                      // most 16-row groups one wave owns
+// 16 bytes per lane from the buffer straight to LDS byte lds_addr + 16 * lane (out-of-range lanes store zeros).
+// Inline assembly: completion is tracked by hand with wait_vmcnt, the compiler does not count these.
+__device__ __forceinline__ void dma16(intx4 rsrc, unsigned lds_addr, int voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voff), "s"(rsrc)
+                 : "memory", "m0");
+}
 
-__global__ __launch_bounds__(64 * MWPB) void helix_gemv_f16_mfma_kernel(const Params p) {
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+__device__ __forceinline__ void wait_steps_in_flight(int steps) {   // at most `steps` later steps' copies pending
+    if (steps >= 3) wait_vmcnt<(SAHEAD >= 3 ? 3 : 0) * SCOPIES>();
+    else if (steps == 2) wait_vmcnt<(SAHEAD >= 2 ? 2 : 0) * SCOPIES>();
+    else if (steps == 1) wait_vmcnt<SCOPIES>();
+    else wait_vmcnt<0>();
+}
+
+__global__ __launch_bounds__(64 * SWPB) void helix_gemv_f16_mfma_stream_kernel(const Params p) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, q = lane >> 4;
     const int m0 = blockIdx.y * 16;
-    const int k_begin = (int)blockIdx.z * p.kchunk;                 // K range of this workgroup: a multiple of MSTEP
+    const int k_begin = (int)blockIdx.z * p.kchunk;                 // K range of this workgroup: a multiple of SXC
     const int k_end = (k_begin + p.kchunk) < p.K ? (k_begin + p.kchunk) : p.K;
-    constexpr int XC = MFMA_KCHUNK_MAX;                              // columns staged at a time
-    constexpr int xrow = XC * 2 + XROW_PAD;                          // bytes per staged activation row
 
     const int ngroups = (p.N + 15) / 16;
-    const int group_first = (blockIdx.x * MWPB + wave) * p.rows_per_wave;      // in units of 16-row groups
+    const int group_first = (blockIdx.x * SWPB + wave) * p.rows_per_wave;      // in units of 16-row groups
     const int group_last = (group_first + p.rows_per_wave) < ngroups ? (group_first + p.rows_per_wave) : ngroups;
+    const int ng = group_last > group_first ? group_last - group_first : 0;   // groups of this wave
 
-    // weights of 16-row group g: load c of a step reads, in lane (r, q), columns 32*c + 8*q .. +7 of row r -- one
-    // instruction covers 64 contiguous bytes of each of 16 rows, the eight loads of a step 512 contiguous bytes
-    // per row.  Rows beyond N read as zeros (buffer bounds).
-    auto w_rsrc = [&](int g) -> __amdgpu_buffer_rsrc_t {
-        const int n0 = g * 16;
-        const int rows_w = (p.N - n0) < 16 ? (p.N - n0) : 16;
-        return __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(p.B + (size_t)n0 * p.ldb), 0,
-                                                 (int)(((size_t)(rows_w - 1) * p.ldb + p.K) * 2), 0x00020000);
+    // ---- the wave's ring and its copy geometry -------------------------------------------------------------------
+    unsigned char* ring = smem + SX_BYTES + wave * (SRING * SSLOT_BYTES);
+    const unsigned ring_lds = (unsigned)(uintptr_t)(lds_ptr_t)ring;
+    // copy instruction i of a step: lanes 0..31 row 2i, lanes 32..63 row 2i + 1; lane position pos = lane % 32 of the
+    // row's 512 bytes holds chunk pos ^ row
+    const int crow = lane >> 5, cpos = lane & 31;
+    int cvoff[SCOPIES], cch[SCOPIES];
+#pragma unroll
+    for (int i = 0; i < SCOPIES; i++) {
+        const int row = 2 * i + crow;
+        cch[i] = cpos ^ row;
+        cvoff[i] = (row * p.ldb + cch[i] * 8) * 2;
+    }
+    // steps in stream order: for every activation chunk, for every group of the wave, the chunk's steps
+    struct Cursor { int kc, gi, k; };
+    auto chunk_end = [&](int kc) -> int { return (kc + SXC) < k_end ? (kc + SXC) : k_end; };
+    auto advance = [&](Cursor& c) {
+        c.k += SSTEP;
+        if (c.k >= chunk_end(c.kc)) {
+            c.gi += 1;
+            if (c.gi >= ng) { c.gi = 0; c.kc += SXC; }
+            c.k = c.kc;
+        }
     };
-    const int woff = (r * p.ldb + 8 * q) * 2;
-    const unsigned char* xl = smem + r * xrow + 8 * q * 2;           // this lane's activation row and column base
+    auto copy_step = [&](const Cursor& c, int slot) {
+        const int n0 = (group_first + c.gi) * 16;
+        const int rows_w = (p.N - n0) < 16 ? (p.N - n0) : 16;
+        const intx4 rw = raw_rsrc(p.B + (size_t)n0 * p.ldb + c.k, (unsigned)(((size_t)(rows_w - 1) * p.ldb + (p.K - c.k)) * 2));
+        const unsigned dst = ring_lds + (unsigned)(slot * SSLOT_BYTES);
+        const int width = k_end - c.k;                       // columns of this step inside the K range
+        if (width >= SSTEP) {
+#pragma unroll
+            for (int i = 0; i < SCOPIES; i++) dma16(rw, dst + i * 1024, cvoff[i]);
+        } else {                                             // partial step: columns beyond the range store zeros
+#pragma unroll
+            for (int i = 0; i < SCOPIES; i++) dma16(rw, dst + i * 1024, cch[i] * 8 < width ? cvoff[i] : 0x7fffffff);
+        }
+    };
 
+    const int nchunks = (k_end - k_begin + SXC - 1) / SXC;
+    // steps of the whole stream of this wave
+    int total_steps = 0;
+    if (ng > 0 && nchunks > 0) {
+        const int last_w = k_end - (k_begin + (nchunks - 1) * SXC);
+        total_steps = ng * ((nchunks - 1) * (SXC / SSTEP) + (last_w + SSTEP - 1) / SSTEP);
+    }
+    Cursor pf{k_begin, 0, k_begin};       // next step to copy
+    int issued = 0, used = 0;
+#pragma unroll 1
+    for (; issued < SAHEAD && issued < total_steps; issued++) {
+        copy_step(pf, issued % SRING);
+        advance(pf);
+    }
+
+    const unsigned char* xl = smem + r * SXROW + 8 * q * 2;          // this lane's activation row and column base
+    const unsigned char* wl = ring + r * (SSTEP * 2);                // this lane's weight row inside a slot
     floatx4 acc[MGROUPS];
 #pragma unroll
     for (int gi = 0; gi < MGROUPS; gi++) acc[gi] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-    // The K range is walked in chunks of XC columns: the workgroup stages 16 activation rows of the chunk in
-    // LDS, then every wave streams the chunk's columns of each of its row groups.
-    for (int kc = k_begin; kc < k_end; kc += XC) {
-        const int ce = (kc + XC) < k_end ? (kc + XC) : k_end;
+    for (int kc = k_begin; kc < k_end; kc += SXC) {
+        const int ce = chunk_end(kc);
         __syncthreads();                                              // the previous chunk has been read
         {
-            constexpr int chunks_per_row = XC / 8;
+            constexpr int chunks_per_row = SXC / 8;
             constexpr int total = 16 * chunks_per_row;
-            for (int c = tid; c < total; c += 64 * MWPB) {
+            for (int c = tid; c < total; c += 64 * SWPB) {
                 const int m = c / chunks_per_row, kk = (c % chunks_per_row) * 8;
                 intx4 v = {0, 0, 0, 0};
                 if (m0 + m < p.M && kc + kk < ce) v = *(const intx4*)(p.A + (size_t)(m0 + m) * p.lda + kc + kk);
-                *(intx4*)(smem + m * xrow + kk * 2) = v;
+                *(intx4*)(smem + m * SXROW + kk * 2) = v;
             }
         }
         __syncthreads();
-
 #pragma unroll
         for (int gi = 0; gi < MGROUPS; gi++) {
-            const int g = group_first + gi;
-            if (g >= group_last) break;
-            const __amdgpu_buffer_rsrc_t rw = w_rsrc(g);
-            half8 wa[MCH], wb[MCH];
-            auto load_step = [&](half8 (&w)[MCH], int k) {
-                if (k + MSTEP <= ce) {
-#pragma unroll
-                    for (int c = 0; c < MCH; c++) w[c] = buf_load8(rw, woff + c * 64, k * 2);
-                } else {   // partial step: columns beyond the chunk read zeros
-#pragma unroll
-                    for (int c = 0; c < MCH; c++)
-                        w[c] = buf_load8(rw, (k + 32 * c + 8 * q < ce) ? woff + c * 64 : 0x7fffffff, k * 2);
+            if (gi >= ng) break;
+            for (int k = kc; k < ce; k += SSTEP) {
+                // keep the stream SAHEAD steps ahead: the slot being refilled is the one the previous step read
+                if (issued < total_steps) {
+                    copy_step(pf, issued % SRING);
+                    advance(pf);
+                    issued++;
                 }
-            };
-            auto mfma_step = [&](const half8 (&w)[MCH], int k) {
+                wait_steps_in_flight(issued - used - 1);
+                const unsigned char* ws = wl + (used % SRING) * SSLOT_BYTES;
 #pragma unroll
-                for (int c = 0; c < MCH; c++) {
+                for (int c = 0; c < SSTEP / 32; c++) {
+                    const half8 wv = *(const half8*)(ws + (((4 * c + q) ^ r) << 4));
                     const half8 xv = *(const half8*)(xl + (k - kc) * 2 + c * 64);
-                    acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(w[c], xv, acc[gi], 0, 0, 0);
+                    acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xv, acc[gi], 0, 0, 0);
                 }
-            };
-            // double-buffered steps: step s+1 is requested before the MFMAs of step s
-            load_step(wa, kc);
-            int k = kc;
-            for (; k + 2 * MSTEP < ce; k += 2 * MSTEP) {
-                load_step(wb, k + MSTEP);
-                mfma_step(wa, k);
-                load_step(wa, k + 2 * MSTEP);
-                mfma_step(wb, k + MSTEP);
-            }
-            if (k + MSTEP < ce) {
-                load_step(wb, k + MSTEP);
-                mfma_step(wa, k);
-                mfma_step(wb, k + MSTEP);
-            } else {
-                mfma_step(wa, k);
+                used++;
             }
         }
     }
@@ -440,9 +498,8 @@ __global__ __launch_bounds__(64 * MWPB) void helix_gemv_f16_mfma_kernel(const Pa
     // lane l holds y[m0 + l % 16][n0 + 4*(l/16) + {0..3}] of each of its groups
 #pragma unroll
     for (int gi = 0; gi < MGROUPS; gi++) {
-        const int g = group_first + gi;
-        if (g >= group_last) break;
-        const int m = m0 + r, n = g * 16 + 4 * q;
+        if (gi >= ng) break;
+        const int m = m0 + r, n = (group_first + gi) * 16 + 4 * q;
         if (m < p.M && n < p.N) {
             if (p.ksplit > 1) {
                 float* dst = p.ws + ((size_t)blockIdx.z * p.M + m) * p.N + n;
@@ -504,24 +561,46 @@ inline const char* info_json() {
 constexpr int mtile_of(int M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
 // K partitioning: enough ranges that M_TILE activation rows of one range fit X_LDS_BYTES_WIDE, at least SPLIT_K
-// MFMA variant: K is partitioned only to give the launch enough waves (one wave owns up to MGROUPS groups of
-// 16 weight rows): ranges are multiples of 256, at least 1024 wide, at least SPLIT_K of them
-inline void k_partition_mfma(int N, int K, int* kchunk, int* ksplit) {
-    const int steps = (K + MSTEP - 1) / MSTEP;
+// LDS-streamed MFMA variant: one workgroup of four waves per compute unit, a wave owns up to MGROUPS groups of 16
+// weight rows; K is partitioned (ranges of whole activation chunks, at least two) only while that brings the launch
+// closer to STREAM_TARGET_WAVES waves
+// Work split of the LDS-streamed variant: g 16-row groups per wave (1 .. MGROUPS) and s K ranges (whole activation
+// chunks, at least two per range).  A launch runs ceil(waves / STREAM_TARGET_WAVES) rounds of waves that each stream
+// g groups x K / s columns; the pair with the shortest rounds x stream wins.  Unit: one wave streaming 16 rows x 512
+// columns (16 KiB, about 2.9 us when 1024 waves share the HBM rate); a round costs about one unit of ramp, a K
+// partition about three for its second kernel.
+inline void stream_split(int N, int K, int* gpw_out, int* split_out) {
+    const int chunks = (K + SXC - 1) / SXC;
     const long long groups = (N + 15) / 16;
-    long long split = (MFMA_TARGET_WAVES / 2 + groups - 1) / groups;     // aim for half the target before splitting
-    const long long max_split = steps / 4 > 1 ? steps / 4 : 1;
-    if (split > max_split) split = max_split;
-    if (split < SPLITK) split = SPLITK;
-    if (split > steps) split = steps;
-    if (split < 1) split = 1;
-    const int per = (int)((steps + split - 1) / split);
-    *kchunk = per * MSTEP;
-    *ksplit = (steps + per - 1) / per;
+    double best = 0.0;
+    int best_g = 1, best_s = 1;
+    for (int s = SPLITK > 1 ? SPLITK : 1; s <= 8; s++) {
+        if (s > 1 && chunks / s < 2) break;
+        const int per = (chunks + s - 1) / s;
+        const int ranges = (chunks + per - 1) / per;
+        for (int g = 1; g <= MGROUPS; g++) {
+            const long long waves = ((groups + g - 1) / g) * ranges;
+            const long long rounds = (waves + STREAM_TARGET_WAVES - 1) / STREAM_TARGET_WAVES;
+            const double unit = SXC / 512.0;
+            const double t = (double)rounds * g * per * unit + (ranges > 1 ? 3.0 : 0.0) + 1.0 * rounds;
+            if (best == 0.0 || t < best) { best = t; best_g = g; best_s = s; }
+        }
+    }
+    *gpw_out = best_g;
+    *split_out = best_s;
+}
+
+inline void k_partition_stream(int N, int K, int* kchunk, int* ksplit) {
+    const int chunks = (K + SXC - 1) / SXC;
+    int g, split;
+    stream_split(N, K, &g, &split);
+    const int per = (chunks + split - 1) / split;
+    *kchunk = per * SXC;
+    *ksplit = (chunks + per - 1) / per;
 }
 
 inline void k_partition(int M, int N, int K, int* kchunk, int* ksplit) {
-    if (M >= MFMA_MIN_M) return k_partition_mfma(N, K, kchunk, ksplit);
+    if (M >= MFMA_MIN_M) return k_partition_stream(N, K, kchunk, ksplit);
     const int mt = mtile_of(M);
     const int steps = (K + KSTEP - 1) / KSTEP;
     int max_steps = X_LDS_BYTES_WIDE / (mt * KSTEP * 2);
@@ -567,19 +646,18 @@ inline int launch_cfg(Params p, hipStream_t s) {
     return launch_waves<MT, ROWS, KU, WPB>(p, lds, s);
 }
 
-inline int launch_mfma(Params p, hipStream_t s) {
+inline int launch_mfma_stream(Params p, hipStream_t s) {
     if ((long long)16 * p.ldb * 2 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
     const long long groups = (p.N + 15) / 16;
-    // 16-row groups per wave: as many (up to MGROUPS) as keep the launch near MFMA_TARGET_WAVES waves; the
-    // staged activations are shared by all groups a workgroup walks
-    long long gpw = (groups * p.ksplit + MFMA_TARGET_WAVES - 1) / MFMA_TARGET_WAVES;
-    if (gpw < 1) gpw = 1;
-    if (gpw > MGROUPS) gpw = MGROUPS;
-    p.rows_per_wave = (int)gpw;
+    int gpw, split;
+    stream_split(p.N, p.K, &gpw, &split);
+    p.rows_per_wave = gpw;
     const long long waves = (groups + gpw - 1) / gpw;
-    const int lds = 16 * (MFMA_KCHUNK_MAX * 2 + XROW_PAD);
-    dim3 grid((unsigned)((waves + MWPB - 1) / MWPB), (p.M + 15) / 16, p.ksplit), block(64 * MWPB);
-    hipLaunchKernelGGL(helix_gemv_f16_mfma_kernel, grid, block, lds, s, p);
+    static int attr_rc = (int)hipFuncSetAttribute((const void*)helix_gemv_f16_mfma_stream_kernel,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, STREAM_LDS_BYTES);
+    if (attr_rc) return attr_rc;
+    dim3 grid((unsigned)((waves + SWPB - 1) / SWPB), (p.M + 15) / 16, p.ksplit), block(64 * SWPB);
+    hipLaunchKernelGGL(helix_gemv_f16_mfma_stream_kernel, grid, block, STREAM_LDS_BYTES, s, p);
     return (int)hipGetLastError();
 }
 
@@ -598,7 +676,7 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     int rc;
     // activation-row tile, like the reference's N_TILE pick from the skinny extent (gemv.cu:232-250); wider
     // tiles take more weight rows per pass so that one LDS read of the activations feeds several rows
-    if (M >= MFMA_MIN_M) rc = launch_mfma(p, s);
+    if (M >= MFMA_MIN_M) rc = launch_mfma_stream(p, s);
     else switch (mtile_of(M)) {
         case 1: rc = launch_cfg<1, GEMV_R1, GEMV_KU1>(p, s); break;
         case 2: rc = launch_cfg<2, GEMV_R2, GEMV_KU2>(p, s); break;

@@ -146,10 +146,12 @@ def test_fp16_cost_model_hand_cases():
         g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 4096 * 4, 4096, K) * 0.99
     # GEMV rows: blocks = ceil(small / row tile) * ceil(big / 128), proportional share of a 256-block round
     gemv = (0, 4, 128, 0, 0, 0, 0)
+    # of the part of the profiled launch beyond one launch's fixed time (GEMV_LAUNCH_FLOOR_S)
+    fixed, stream = g16.GEMV_LAUNCH_FLOOR_S, 2.56e-3 - g16.GEMV_LAUNCH_FLOOR_S
     assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 256, K) == pytest.approx(2.56e-3)
-    assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 128, K) == pytest.approx(1.28e-3)
+    assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 128, K) == pytest.approx(fixed + stream / 2)
     assert g16.config_cost(gemv, 2.56e-3, 128 * 256, 3, K) == pytest.approx(2.56e-3)      # operands swap
-    assert g16.config_cost(gemv, 2.56e-3, 16, 128 * 256, K) == pytest.approx(4 * 2.56e-3)
+    assert g16.config_cost(gemv, 2.56e-3, 16, 128 * 256, K) == pytest.approx(fixed + 4 * stream)
     assert g16.config_cost(gemv, 1e-9, 1, 128, 512) == g16.GEMV_LAUNCH_FLOOR_S
     # conv never selects a GEMV row
     d2 = dict(d)
@@ -192,7 +194,7 @@ def test_fp16_cost_model_two_point_profile():
     r_small, r_big = g16.round_time(17e-6, 4e-6, 64), g16.round_time(60e-6, 8e-6, 64)
     assert c_small == pytest.approx(49 * r_small - 48 * g16.ROUND_OVERLAP_S)
     assert c_big == pytest.approx(max(4 * r_big - 3 * g16.ROUND_OVERLAP_S,
-                                      roofline.gemm_bytes(100352, 256, 64, 2) / (g16.HBM_SUSTAINED_FRACTION * roofline.HBM_BYTES_PER_S)))
+                                      roofline.gemm_bytes(100352, 256, 64, 2) / (g16.TILE_HBM_SUSTAINED_FRACTION * roofline.HBM_BYTES_PER_S)))
     assert g16.cost_model(d, 100352, 256, 64) == big
     # without the short point a round is taken to cost K / K_profile of the profiled one: 49 almost free rounds
     assert g16.config_cost(small, d[small], 100352, 256, 64) == pytest.approx(49 * 17e-6 * 64 / K)
