@@ -20,7 +20,7 @@ HBM_SUSTAINED_FRACTION = 0.8  # share of the datasheet HBM rate a streaming kern
 # the weight-streaming kernels, whose profile point is cold
 TILE_HBM_SUSTAINED_FRACTION = 0.68
 GEMV_LAUNCH_FLOOR_S = 3.4e-6       # a kernel launch on an idle queue; keeps tiny problems from looking free
-GEMV_MFMA_FLOOR_S = 6.5e-6         # 9 or more activation rows: the K-partitioned MFMA variant plus its reduction
+GEMV_MFMA_FLOOR_S = 4.4e-6         # 9 or more activation rows: the LDS-streamed MFMA variant (staging + cross-wave sum)
 GEMV_MFMA_MIN_M = 9                # MFMA_MIN_M of src_template/MI355X_FP16/gemv.hip
 # the weight-streaming kernels pass over the weights once per 16 activation rows: beyond one pass a tile kernel,
 # which reads them once per BLOCK_ROWS rows, is the better streamer, and the per-round share the model assumes

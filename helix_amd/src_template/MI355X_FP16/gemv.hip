@@ -31,18 +31,21 @@
 //     atomics, gemv_splitK.cu:213-217).
 //
 // MFMA variant (M >= MFMA_MIN_M)
-//   * a workgroup (four waves, one per compute unit) walks its K range in chunks of 512 columns and stages 16
-//     activation rows of the chunk in LDS, rows 16 bytes apart from a multiple of 256 so that 16 rows of one column
-//     sit in 16 different bank groups;
-//   * a wave owns runs of 16 consecutive weight rows and streams them through a ring in LDS that is private to it:
+//   * a workgroup (four waves, one per compute unit) walks its K range in chunks of 512 or 1024 columns and stages
+//     16 activation rows of the chunk in LDS, 16-byte chunks XOR-swizzled with the row so that the 16 rows of one
+//     column sit in 16 different bank groups;
+//   * weights stream in steps of 16 consecutive rows x 256 columns through a ring in LDS that is private to a wave:
 //     every copy instruction (buffer_load ... lds) fetches 512 contiguous bytes of each of two rows -- whole-row
 //     spans, the pattern that streams fastest -- and the MFMA operands (lane l: row l % 16, columns 8*(l/16) .. +7 of
 //     a 32-wide block) are read back from LDS.  Loading the operand layout straight into registers (16 rows x 64
 //     bytes per instruction) measured 4.3 TB/s on 8192 x 28672 weights at 16 rows, this variant 5.3;
-//   * eight MFMAs per 256-column step accumulate the 16 x 16 block y[m][n]; copies run three steps ahead; buffer
-//     bounds checking zero-fills weight rows beyond N;
-//   * groups per wave and K ranges (blockIdx.z; FP32 workspace + fixed-order reduce) are chosen per problem so that
-//     rounds of 1024 waves x the stream of one wave is shortest (stream_split).
+//   * eight MFMAs per step accumulate the 16 x 16 block y[m][n]; copies run three steps ahead; buffer bounds
+//     checking zero-fills weight rows beyond N;
+//   * two work splits: a wave owns its own row groups and all columns of the K range, or the four waves of a
+//     workgroup share their groups, take a quarter of every staged chunk each and add their sums through LDS at the
+//     end (four times the waves for short streams, no second kernel);
+//   * split, groups per owner and K ranges (blockIdx.z; FP32 workspace + fixed-order reduce) are chosen per problem
+//     so that rounds of 1024 waves x the stream of one wave is shortest (stream_split).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -347,13 +350,21 @@ constexpr int SRING = STREAM_RING;               // ring slots per wave
 constexpr int SAHEAD = SRING - 1;                // steps a copy is issued ahead of its use
 constexpr int SSLOT_BYTES = 16 * SSTEP * 2;      // 8 KiB: 16 rows x 512 bytes
 constexpr int SCOPIES = SSLOT_BYTES / 1024;      // copy instructions per step (8): two rows each
-constexpr int SXC = STREAM_XC;                   // activation columns staged at a time
 constexpr int SWPB = 4;                          // waves per workgroup
-constexpr int SXROW = SXC * 2 + XROW_PAD;        // bytes per staged activation row
-constexpr int SX_BYTES = ((16 * SXROW + 1023) / 1024) * 1024;
-constexpr int STREAM_LDS_BYTES = SX_BYTES + SWPB * SRING * SSLOT_BYTES;
-static_assert(STREAM_LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
+// Two work splits.  KW = 1: every wave owns its own 16-row groups and runs over the whole K range of the workgroup;
+// STREAM_XC activation columns are staged at a time.  KW = SWPB: the waves of a workgroup share their groups and
+// split every staged chunk of SWPB * SSTEP columns between them, one step each, and add their partial sums through
+// LDS at the end -- four times the waves for the same number of rows without a second kernel, which is what short
+// streams (a few thousand rows) need.
+constexpr int stream_xc(int kw) { return kw == 1 ? STREAM_XC : kw * SSTEP; }
+// staged activations: 16 rows of xc columns; the 16-byte chunk ch of row m sits at chunk position ch ^ m of its row
+// (rows are a multiple of 256 bytes apart, so unswizzled the 16 rows of one column would share their banks)
+constexpr int stream_x_bytes(int kw) { return 16 * stream_xc(kw) * 2; }
+constexpr int stream_lds_bytes(int kw) { return stream_x_bytes(kw) + SWPB * SRING * SSLOT_BYTES; }
+static_assert(stream_lds_bytes(1) <= 160 * 1024 && stream_lds_bytes(SWPB) <= 160 * 1024,
+              "LDS budget of a gfx950 CU exceeded");
 static_assert(SAHEAD * SCOPIES <= 63, "copies in flight are counted in a 6-bit counter");
+static_assert(STREAM_XC % SSTEP == 0 && STREAM_XC >= SSTEP, "a staged chunk is whole steps");
 
 typedef __attribute__((address_space(3))) unsigned char* lds_ptr_t;
 
@@ -376,14 +387,31 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
 }
-__device__ __forceinline__ void wait_steps_in_flight(int steps) {   // at most `steps` later steps' copies pending
-    if (steps >= 3) wait_vmcnt<(SAHEAD >= 3 ? 3 : 0) * SCOPIES>();
-    else if (steps == 2) wait_vmcnt<(SAHEAD >= 2 ? 2 : 0) * SCOPIES>();
-    else if (steps == 1) wait_vmcnt<SCOPIES>();
-    else wait_vmcnt<0>();
+// At most `steps` later steps' copies (SCOPIES instructions each) plus `extra` other loads may still be pending.
+template <int EXTRA>
+__device__ __forceinline__ void wait_steps_in_flight(int steps) {
+    if (steps >= 3) wait_vmcnt<(SAHEAD >= 3 ? 3 : 0) * SCOPIES + (SAHEAD >= 3 ? EXTRA : 0)>();
+    else if (steps == 2) wait_vmcnt<(SAHEAD >= 2 ? 2 : 0) * SCOPIES + (SAHEAD >= 2 ? EXTRA : 0)>();
+    else if (steps == 1) wait_vmcnt<SCOPIES + EXTRA>();
+    else wait_vmcnt<EXTRA>();
 }
 
+// 16 bytes per lane from the buffer into registers, issued from inline assembly for the same reason as dma16: the
+// compiler would put s_waitcnt vmcnt(0) in front of the first use and drain the weight copies in flight with it.
+// The value is valid only behind a hand-placed wait; x_landed ties the registers to that wait.
+__device__ __forceinline__ intx4 load16_untracked(intx4 rsrc, int voff) {
+    intx4 v;
+    asm volatile("buffer_load_dwordx4 %0, %1, %2, 0 offen" : "=v"(v) : "v"(voff), "s"(rsrc) : "memory");
+    return v;
+}
+__device__ __forceinline__ void x_landed(intx4& v) { asm volatile("" : "+v"(v) : : "memory"); }
+
+template <int KW>
 __global__ __launch_bounds__(64 * SWPB) void helix_gemv_f16_mfma_stream_kernel(const Params p) {
+    constexpr int SXC = stream_xc(KW);               // activation columns staged at a time
+    constexpr int SUB = SXC / KW;                    // columns of a staged chunk that one wave works on
+    constexpr int SXROW = SXC * 2;                   // bytes per staged activation row
+    constexpr int SX_BYTES = stream_x_bytes(KW);
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -394,7 +422,7 @@ __global__ __launch_bounds__(64 * SWPB) void helix_gemv_f16_mfma_stream_kernel(c
     const int k_end = (k_begin + p.kchunk) < p.K ? (k_begin + p.kchunk) : p.K;
 
     const int ngroups = (p.N + 15) / 16;
-    const int group_first = (blockIdx.x * SWPB + wave) * p.rows_per_wave;      // in units of 16-row groups
+    const int group_first = (KW == 1 ? blockIdx.x * SWPB + wave : blockIdx.x) * p.rows_per_wave;   // 16-row groups
     const int group_last = (group_first + p.rows_per_wave) < ngroups ? (group_first + p.rows_per_wave) : ngroups;
     const int ng = group_last > group_first ? group_last - group_first : 0;   // groups of this wave
 
@@ -411,15 +439,21 @@ __global__ __launch_bounds__(64 * SWPB) void helix_gemv_f16_mfma_stream_kernel(c
         cch[i] = cpos ^ row;
         cvoff[i] = (row * p.ldb + cch[i] * 8) * 2;
     }
-    // steps in stream order: for every activation chunk, for every group of the wave, the chunk's steps
+    // steps in stream order: for every activation chunk, for every group of the wave, the steps of the wave's share
+    // [sub_begin, sub_end) of the chunk (the whole chunk when KW = 1; empty only in the last chunk of the range)
     struct Cursor { int kc, gi, k; };
     auto chunk_end = [&](int kc) -> int { return (kc + SXC) < k_end ? (kc + SXC) : k_end; };
+    auto sub_begin = [&](int kc) -> int { return KW == 1 ? kc : kc + wave * SUB; };
+    auto sub_end = [&](int kc) -> int {
+        const int e = KW == 1 ? kc + SXC : kc + (wave + 1) * SUB;
+        return e < k_end ? e : k_end;
+    };
     auto advance = [&](Cursor& c) {
         c.k += SSTEP;
-        if (c.k >= chunk_end(c.kc)) {
+        if (c.k >= sub_end(c.kc)) {
             c.gi += 1;
             if (c.gi >= ng) { c.gi = 0; c.kc += SXC; }
-            c.k = c.kc;
+            c.k = sub_begin(c.kc);
         }
     };
     auto copy_step = [&](const Cursor& c, int slot) {
@@ -437,57 +471,86 @@ __global__ __launch_bounds__(64 * SWPB) void helix_gemv_f16_mfma_stream_kernel(c
         }
     };
 
-    const int nchunks = (k_end - k_begin + SXC - 1) / SXC;
     // steps of the whole stream of this wave
     int total_steps = 0;
-    if (ng > 0 && nchunks > 0) {
-        const int last_w = k_end - (k_begin + (nchunks - 1) * SXC);
-        total_steps = ng * ((nchunks - 1) * (SXC / SSTEP) + (last_w + SSTEP - 1) / SSTEP);
+#pragma unroll 1
+    for (int kc = k_begin; kc < k_end; kc += SXC) {
+        const int w = sub_end(kc) - sub_begin(kc);
+        if (w > 0) total_steps += ng * ((w + SSTEP - 1) / SSTEP);
     }
-    Cursor pf{k_begin, 0, k_begin};       // next step to copy
+    // ---- activations: the next chunk is fetched into registers while the current one is worked on ---------------
+    constexpr int CPR = SXC / 8;                         // 16-byte chunks per staged row
+    constexpr int XPT = 16 * CPR / (64 * SWPB);          // chunks per thread
+    static_assert(16 * CPR % (64 * SWPB) == 0, "the staged chunk divides over the workgroup");
+    static_assert(SAHEAD * SCOPIES + XPT <= 63, "loads in flight are counted in a 6-bit counter");
+    const int rows_a = (p.M - m0) < 16 ? (p.M - m0) : 16;
+    const intx4 rx = raw_rsrc(p.A + (size_t)m0 * p.lda, (unsigned)(((size_t)(rows_a - 1) * p.lda + p.K) * 2));
+    intx4 xr[XPT];
+    auto fetch_x = [&](int kc) {                         // rows beyond M and columns beyond the K range read as zero
+        const int ce = chunk_end(kc);
+#pragma unroll
+        for (int i = 0; i < XPT; i++) {
+            const int c = tid + i * (64 * SWPB);
+            const int m = c / CPR, kk = (c % CPR) * 8;
+            xr[i] = load16_untracked(rx, (m < rows_a && kc + kk < ce) ? (m * p.lda + kc + kk) * 2 : 0x7fffffff);
+        }
+    };
+    int steps_after_x = 0;                               // weight steps issued behind the latest fetch_x
+    if (k_begin < k_end) fetch_x(k_begin);
+
+    Cursor pf{k_begin, 0, sub_begin(k_begin)};       // next step to copy
     int issued = 0, used = 0;
 #pragma unroll 1
     for (; issued < SAHEAD && issued < total_steps; issued++) {
         copy_step(pf, issued % SRING);
         advance(pf);
+        steps_after_x++;
     }
 
-    const unsigned char* xl = smem + r * SXROW + 8 * q * 2;          // this lane's activation row and column base
+    const unsigned char* xl = smem + r * SXROW;                      // this lane's activation row
     const unsigned char* wl = ring + r * (SSTEP * 2);                // this lane's weight row inside a slot
     floatx4 acc[MGROUPS];
 #pragma unroll
     for (int gi = 0; gi < MGROUPS; gi++) acc[gi] = floatx4{0.f, 0.f, 0.f, 0.f};
 
     for (int kc = k_begin; kc < k_end; kc += SXC) {
-        const int ce = chunk_end(kc);
         __syncthreads();                                              // the previous chunk has been read
-        {
-            constexpr int chunks_per_row = SXC / 8;
-            constexpr int total = 16 * chunks_per_row;
-            for (int c = tid; c < total; c += 64 * SWPB) {
-                const int m = c / chunks_per_row, kk = (c % chunks_per_row) * 8;
-                intx4 v = {0, 0, 0, 0};
-                if (m0 + m < p.M && kc + kk < ce) v = *(const intx4*)(p.A + (size_t)(m0 + m) * p.lda + kc + kk);
-                *(intx4*)(smem + m * SXROW + kk * 2) = v;
-            }
+        // loads complete in order: the chunk's activations are older than the steps_after_x newest weight steps
+        wait_steps_in_flight<0>(steps_after_x);
+#pragma unroll
+        for (int i = 0; i < XPT; i++) {
+            const int c = tid + i * (64 * SWPB);
+            const int m = c / CPR, ch = c % CPR;
+            x_landed(xr[i]);
+            *(intx4*)(smem + m * SXROW + ((ch ^ m) << 4)) = xr[i];
         }
         __syncthreads();
+        if (kc + SXC < k_end) {
+            fetch_x(kc + SXC);
+            steps_after_x = 0;
+        } else {
+            steps_after_x = 1 << 20;                                  // nothing but weight steps in flight from here on
+        }
 #pragma unroll
         for (int gi = 0; gi < MGROUPS; gi++) {
             if (gi >= ng) break;
-            for (int k = kc; k < ce; k += SSTEP) {
+            for (int k = sub_begin(kc); k < sub_end(kc); k += SSTEP) {
                 // keep the stream SAHEAD steps ahead: the slot being refilled is the one the previous step read
                 if (issued < total_steps) {
                     copy_step(pf, issued % SRING);
                     advance(pf);
                     issued++;
+                    steps_after_x++;
                 }
-                wait_steps_in_flight(issued - used - 1);
+                // step `used` has landed when only what was issued behind it is pending: the later steps and, if it
+                // was fetched behind that step, the next chunk of activations
+                if (steps_after_x <= issued - used - 1) wait_steps_in_flight<XPT>(issued - used - 1);
+                else wait_steps_in_flight<0>(issued - used - 1);
                 const unsigned char* ws = wl + (used % SRING) * SSLOT_BYTES;
 #pragma unroll
                 for (int c = 0; c < SSTEP / 32; c++) {
                     const half8 wv = *(const half8*)(ws + (((4 * c + q) ^ r) << 4));
-                    const half8 xv = *(const half8*)(xl + (k - kc) * 2 + c * 64);
+                    const half8 xv = *(const half8*)(xl + (((((k - kc) >> 3) + 4 * c + q) ^ r) << 4));
                     acc[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wv, xv, acc[gi], 0, 0, 0);
                 }
                 used++;
@@ -495,10 +558,31 @@ __global__ __launch_bounds__(64 * SWPB) void helix_gemv_f16_mfma_stream_kernel(c
         }
     }
 
+    if (KW > 1) {
+        // the waves hold partial sums of the same groups: wave w parks its sums of every group but those it will
+        // store itself (gi % KW == w) in the activation staging area, then adds the other waves' sums of its own
+        floatx4* park = (floatx4*)smem;               // [wave][group][lane]
+        static_assert(KW == 1 || KW * MGROUPS * 64 * 16 <= stream_x_bytes(KW), "parked sums fit the staging area");
+        __syncthreads();                              // every wave has read its last activations
+#pragma unroll
+        for (int gi = 0; gi < MGROUPS; gi++)
+            if (gi < ng && gi % KW != wave) park[(wave * MGROUPS + gi) * 64 + lane] = acc[gi];
+        __syncthreads();
+#pragma unroll
+        for (int gi = 0; gi < MGROUPS; gi++)
+            if (gi < ng && gi % KW == wave)
+                for (int w = 0; w < KW; w++)
+                    if (w != wave) {
+                        const floatx4 o = park[(w * MGROUPS + gi) * 64 + lane];
+                        acc[gi][0] += o[0]; acc[gi][1] += o[1]; acc[gi][2] += o[2]; acc[gi][3] += o[3];
+                    }
+    }
+
     // lane l holds y[m0 + l % 16][n0 + 4*(l/16) + {0..3}] of each of its groups
 #pragma unroll
     for (int gi = 0; gi < MGROUPS; gi++) {
         if (gi >= ng) break;
+        if (KW > 1 && gi % KW != wave) continue;
         const int m = m0 + r, n = (group_first + gi) * 16 + 4 * q;
         if (m < p.M && n < p.N) {
             if (p.ksplit > 1) {
@@ -560,43 +644,40 @@ inline const char* info_json() {
 
 constexpr int mtile_of(int M) { return M <= 1 ? 1 : M <= 2 ? 2 : M <= 4 ? 4 : M <= 8 ? 8 : 16; }
 
-// K partitioning: enough ranges that M_TILE activation rows of one range fit X_LDS_BYTES_WIDE, at least SPLIT_K
-// LDS-streamed MFMA variant: one workgroup of four waves per compute unit, a wave owns up to MGROUPS groups of 16
-// weight rows; K is partitioned (ranges of whole activation chunks, at least two) only while that brings the launch
-// closer to STREAM_TARGET_WAVES waves
-// Work split of the LDS-streamed variant: g 16-row groups per wave (1 .. MGROUPS) and s K ranges (whole activation
-// chunks, at least two per range).  A launch runs ceil(waves / STREAM_TARGET_WAVES) rounds of waves that each stream
-// g groups x K / s columns; the pair with the shortest rounds x stream wins.  Unit: one wave streaming 16 rows x 512
-// columns (16 KiB, about 2.9 us when 1024 waves share the HBM rate); a round costs about one unit of ramp, a K
-// partition about three for its second kernel.
-inline void stream_split(int N, int K, int* gpw_out, int* split_out) {
-    const int chunks = (K + SXC - 1) / SXC;
+// Work split of the LDS-streamed variant: kw = 1 (a wave owns its groups) or SWPB (the waves of a workgroup share
+// theirs and split the columns), g 16-row groups per wave or workgroup (1 .. MGROUPS) and s K ranges over grid z
+// (whole activation chunks, at least two per range).  A launch runs ceil(waves / STREAM_TARGET_WAVES) rounds of waves
+// that each stream g groups x (K / s) / kw columns; the split with the shortest rounds x stream wins.  Unit: one wave
+// streaming 16 rows x 512 columns (16 KiB, about 2.9 us when 1024 waves share the HBM rate); a round costs about one
+// unit of ramp, a K partition over grid z about three for its second kernel.
+struct StreamSplit { int kw, groups, ranges, kchunk; };
+inline StreamSplit stream_split(int N, int K) {
     const long long groups = (N + 15) / 16;
     double best = 0.0;
-    int best_g = 1, best_s = 1;
-    for (int s = SPLITK > 1 ? SPLITK : 1; s <= 8; s++) {
-        if (s > 1 && chunks / s < 2) break;
-        const int per = (chunks + s - 1) / s;
-        const int ranges = (chunks + per - 1) / per;
-        for (int g = 1; g <= MGROUPS; g++) {
-            const long long waves = ((groups + g - 1) / g) * ranges;
-            const long long rounds = (waves + STREAM_TARGET_WAVES - 1) / STREAM_TARGET_WAVES;
-            const double unit = SXC / 512.0;
-            const double t = (double)rounds * g * per * unit + (ranges > 1 ? 3.0 : 0.0) + 1.0 * rounds;
-            if (best == 0.0 || t < best) { best = t; best_g = g; best_s = s; }
+    StreamSplit pick{1, 1, 1, K};
+    for (int kw = 1; kw <= SWPB; kw += SWPB - 1) {
+        const int xc = stream_xc(kw);
+        const int chunks = (K + xc - 1) / xc;
+        for (int s = SPLITK > 1 ? SPLITK : 1; s <= 8; s++) {
+            if (s > 1 && chunks / s < 2) break;
+            const int per = (chunks + s - 1) / s;
+            const int ranges = (chunks + per - 1) / per;
+            for (int g = 1; g <= MGROUPS; g++) {
+                const long long waves = ((groups + g - 1) / g) * ranges * kw;
+                const long long rounds = (waves + STREAM_TARGET_WAVES - 1) / STREAM_TARGET_WAVES;
+                const double unit = xc / 512.0 / kw;
+                const double t = (double)rounds * g * per * unit + (ranges > 1 ? 3.0 : 0.0) + 1.0 * rounds;
+                if (best == 0.0 || t < best) { best = t; pick = StreamSplit{kw, g, ranges, per * xc}; }
+            }
         }
     }
-    *gpw_out = best_g;
-    *split_out = best_s;
+    return pick;
 }
 
 inline void k_partition_stream(int N, int K, int* kchunk, int* ksplit) {
-    const int chunks = (K + SXC - 1) / SXC;
-    int g, split;
-    stream_split(N, K, &g, &split);
-    const int per = (chunks + split - 1) / split;
-    *kchunk = per * SXC;
-    *ksplit = (chunks + per - 1) / per;
+    const StreamSplit sp = stream_split(N, K);
+    *kchunk = sp.kchunk;
+    *ksplit = sp.ranges;
 }
 
 inline void k_partition(int M, int N, int K, int* kchunk, int* ksplit) {
@@ -646,19 +727,25 @@ inline int launch_cfg(Params p, hipStream_t s) {
     return launch_waves<MT, ROWS, KU, WPB>(p, lds, s);
 }
 
-inline int launch_mfma_stream(Params p, hipStream_t s) {
-    if ((long long)16 * p.ldb * 2 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
-    const long long groups = (p.N + 15) / 16;
-    int gpw, split;
-    stream_split(p.N, p.K, &gpw, &split);
-    p.rows_per_wave = gpw;
-    const long long waves = (groups + gpw - 1) / gpw;
-    static int attr_rc = (int)hipFuncSetAttribute((const void*)helix_gemv_f16_mfma_stream_kernel,
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, STREAM_LDS_BYTES);
+template <int KW>
+inline int launch_mfma_stream_kw(Params p, long long workgroups, hipStream_t s) {
+    static int attr_rc = (int)hipFuncSetAttribute((const void*)helix_gemv_f16_mfma_stream_kernel<KW>,
+                                                  hipFuncAttributeMaxDynamicSharedMemorySize, stream_lds_bytes(KW));
     if (attr_rc) return attr_rc;
-    dim3 grid((unsigned)((waves + SWPB - 1) / SWPB), (p.M + 15) / 16, p.ksplit), block(64 * SWPB);
-    hipLaunchKernelGGL(helix_gemv_f16_mfma_stream_kernel, grid, block, STREAM_LDS_BYTES, s, p);
+    dim3 grid((unsigned)workgroups, (p.M + 15) / 16, p.ksplit), block(64 * SWPB);
+    hipLaunchKernelGGL(helix_gemv_f16_mfma_stream_kernel<KW>, grid, block, stream_lds_bytes(KW), s, p);
     return (int)hipGetLastError();
+}
+
+inline int launch_mfma_stream(Params p, hipStream_t s) {
+    if ((long long)16 * p.ldb * 2 >= 0x7fffffffLL || (long long)16 * p.lda * 2 >= 0x7fffffffLL)
+        return HELIX_ERR_INVALID_VALUE;
+    const long long groups = (p.N + 15) / 16;
+    const StreamSplit sp = stream_split(p.N, p.K);
+    p.rows_per_wave = sp.groups;
+    const long long owners = (groups + sp.groups - 1) / sp.groups;       // waves (kw = 1) or workgroups that own groups
+    if (sp.kw == 1) return launch_mfma_stream_kw<1>(p, (owners + SWPB - 1) / SWPB, s);
+    return launch_mfma_stream_kw<SWPB>(p, owners, s);
 }
 
 inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int lda, int ldb, int ldc, void* ws,

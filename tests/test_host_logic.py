@@ -261,6 +261,30 @@ def test_fp32_cost_model_extra_points():
         pytest.approx(g32.GEMV_LAUNCH_FLOOR_S + g32.GEMV_SPLITK_EXTRA_S)
 
 
+def test_build_records_kernel_resources_and_conv_skips_spilling_gathers(monkeypatch):
+    """hipcc's per-kernel resource remarks are parsed at build time; the conv cost model leaves out configurations
+    whose gather kernel for the layer's channel count spills registers to scratch."""
+    text = (
+        "gemm.hip:144:1: remark: Function Name: _ZN12_GLOBAL__N_121helix_gemm_f16_kernelILi0ELi2ELi256ELi256ELi128ELi64ELi64ELi1EEEvNS_6ParamsE [-Rpass-analysis=kernel-resource-usage]\n"
+        "gemm.hip:144:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]\n"
+        "gemm.hip:144:1: remark:     AGPRs: 0 [-Rpass-analysis=kernel-resource-usage]\n"
+        "gemm.hip:144:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]\n"
+        "gemm.hip:144:1: remark:     Occupancy [waves/SIMD]: 2 [-Rpass-analysis=kernel-resource-usage]\n"
+        "gemm.hip:144:1: remark: Function Name: _ZN12_GLOBAL__N_121helix_gemm_f16_kernelILi2ELi2ELi256ELi256ELi128ELi64ELi64ELi1EEEvNS_6ParamsE [-Rpass-analysis=kernel-resource-usage]\n"
+        "gemm.hip:144:1: remark:     VGPRs: 256 [-Rpass-analysis=kernel-resource-usage]\n"
+        "gemm.hip:144:1: remark:     ScratchSize [bytes/lane]: 52 [-Rpass-analysis=kernel-resource-usage]\n")
+    usage = helix_runtime.parse_resource_usage(text)
+    assert len(usage) == 2
+    gemm_k, conv_k = sorted(usage)
+    assert usage[gemm_k] == {"vgprs": 256, "agprs": 0, "scratch": 0, "occupancy": 2} and usage[conv_k]["scratch"] == 52
+    big, small = (2, 256, 256, 128, 64, 0, 64), (2, 128, 128, 64, 64, 0, 64)
+    d = {big: 1e-9, small: 1.0}
+    monkeypatch.setattr(c16, "kernel_resources", lambda path: usage if "256_256" in path else {})
+    assert c16.conv_kernel_scratch(big, 64) == 52 and c16.conv_kernel_scratch(big, 24) == 0   # mode 2 spills, mode 1 has no record
+    assert c16.cost_model(d, 100352, 256, 64, 64) == small      # the cheaper prediction is skipped: its gather spills
+    assert c16.cost_model(d, 100352, 256, 72, 24) == big
+
+
 def test_fastdiv_header_matches_integer_division(tmp_path):
     """The conv gathers divide by OW, OH, IC and kW with a multiply and a shift (common/helix_fastdiv.h); the
     host half of the header is compiled and swept against `/` here."""
