@@ -20,8 +20,9 @@
 //     at the barrier two phases earlier), and at the end of C(t) it waits until tile t + 1 has landed, so the
 //     barrier behind C(t) publishes tile t + 1 to both groups.  A copy has K_STAGES - 1 K tiles to land.
 // Measured on 8192^3 (256 x 256 tile): with nothing to copy the two-group schedule runs a 64-column K tile in 2190
-// cycles where the MFMAs alone need 2048; a burst of 64 KiB of copies per compute unit takes 1.4 us to land, which
-// is why the ring is built from 32-column stages for that tile (four stages: three tiles in flight).
+// cycles where the MFMAs alone need 2048; a burst of 64 KiB of copies per compute unit takes 1.4 us to land.  Two
+// 64-column stages measure fastest for that tile; rings of three or four 32-column stages (two or three tiles in
+// flight, but twice the barriers per K) are about 10 % slower there and are built for the smaller tiles.
 //
 // LDS layout: rows of 128 bytes (256 for BLOCK_K = 128); 16-byte chunk c of LDS row r sits at chunk position
 // c ^ key(r), key(r) = (r / rows_per_256B) mod chunks_per_row, the layout gemm.hip reads without bank conflicts.
