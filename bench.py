@@ -126,8 +126,8 @@ def engine_clock_mhz(run_for_s, work):
 def cpu_baseline(budget_s=24.0):
     """The reference's x86_CPU path (restated in oracle/) on this machine's host cores: two-phase
     profile, tiling pick, then the packed / n-parallel schedule.  The headline sample is FP32 2048^3 (the
-    largest square the host finishes a few times within the budget); two more samples cover configuration 1
-    (FP32 1024^3, U[-1,1)) and one BERT-base GEMM (4096 x 768 x 768, FP32)."""
+    largest square the host finishes a few times within the budget); three more samples cover configuration 1
+    (FP32 1024^3), one convolution layer of configuration 4 and one BERT-base GEMM of configuration 5."""
     import numpy as np
     from oracle import oracle as O
     cores = os.cpu_count() or 1
@@ -143,11 +143,15 @@ def cpu_baseline(budget_s=24.0):
 
     left = max(budget_s - prof_s, 6.0)
     s = 2048
-    cost, gflops, padded, tiling, number = sample(s, s, s, 0.6 * left)
+    cost, gflops, padded, tiling, number = sample(s, s, s, 0.5 * left)
     extra = []
+    # the reference's x86 path times a convolution as the GEMM of its im2col extents (restated in the oracle)
+    conv_layer = (32, 128, 28, 28, 128, 3, 3, 1, 1)
     for (label, (M, N, K)) in (("config 1: FP32 GEMM 1024^3", (1024, 1024, 1024)),
+                               ("config 4: conv 28x28x128 3x3 batch 32 as its im2col GEMM, FP32",
+                                O.x86_conv_gemm_extents(*conv_layer)),
                                ("config 5: BERT-base FFN-out GEMM 4096x768x3072, FP32", (4096, 768, 3072))):
-        c, g, pd, tl, n = sample(M, N, K, 0.2 * left)
+        c, g, pd, tl, n = sample(M, N, K, 0.15 * left)
         extra.append({"sample": f"{label} (padded to {pd[0]}x{pd[1]}x{pd[2]}), tiling {tl}, mean of {n} runs",
                       "value": round(g / 1e3, 4), "unit": "TFLOP/s", "ms": round(c * 1e3, 3)})
     return {"value": round(gflops / 1e3, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",

@@ -8,6 +8,9 @@ Reference files restated here (paths relative to the reference checkout):
   scripts/x86_CPU/profile_x86_CPU.py:62-122          two-phase register-block / cache-block profile
   scripts/x86_CPU/benchmark_x86_CPU_gemm.py:46-68    get_tiling
   scripts/x86_CPU/benchmark_x86_CPU_gemm.py:71-136   sch_gemm (padding) + get_Helix_result (timing)
+  scripts/x86_CPU/changed_profile_x86_CPU.py:62-127  the profile whose cache blocks are timed, not extrapolated
+  scripts/x86_CPU/benchmark_x86_CPU_conv.py:119-140  convolution = the GEMM of its im2col extents
+  scripts/x86_CPU/benchmark_x86_CPU_model_level_LLM.py:119-135, :180-195  per-GEMM seconds summed over a model's list
 """
 import ctypes
 import math
@@ -232,14 +235,17 @@ def x86_register_blocks():
     return out
 
 
-def x86_profile(peak_gflops=X86_PEAK_GFLOPS, number=1000, time_fn=None, keep=0.6):
+def x86_profile(peak_gflops=X86_PEAK_GFLOPS, number=1000, time_fn=None, keep=0.6, timed_cache_blocks=False):
     """Two-phase profile (profile_x86_CPU.py:62-118): time every register block on a
     (20*M1*M2) x (16*N1*N2) x (16*K1) problem, keep those above `keep`*peak, then extrapolate cache
     blocks up to 256 x 256.  Returns (register_block_dict, cache_block_dict).
 
     `time_fn(M,N,K,m1,m2,n1,n2,k1) -> seconds` may be injected (tests use a deterministic one).
     `peak_gflops=None` calibrates the peak to the fastest measured register block, for hosts
-    whose core is not the Skylake-AVX512 the constant 153 presumes."""
+    whose core is not the Skylake-AVX512 the constant 153 presumes.
+    `timed_cache_blocks=True` is changed_profile_x86_CPU.py:62-127: the only difference (its lines 110-119
+    against profile_x86_CPU.py:110) is that every cache block is run and timed with the profile-time
+    schedule of its register block instead of being priced as a multiple of the register block's time."""
     L = lib()
     rng = np.random.default_rng(0)
     measured = {}
@@ -271,7 +277,16 @@ def x86_profile(peak_gflops=X86_PEAK_GFLOPS, number=1000, time_fn=None, keep=0.6
                 M = Mx * M1 * M2
                 N = Nx * N1 * N2
                 K = 16 * K1
-                cost = value[0] / (20 * 16) * (Mx * Nx)
+                if not timed_cache_blocks:
+                    cost = value[0] / (20 * 16) * (Mx * Nx)
+                elif time_fn is not None:
+                    cost = time_fn(M, N, K, M1, M2, N1, N2, K1)
+                else:
+                    A = rng.random((M, K), dtype=np.float32)
+                    B = rng.random((K, N), dtype=np.float32)
+                    C = np.zeros((M, N), dtype=np.float32)
+                    cost = L.oracle_x86_time_profile_kernel(A.ctypes.data_as(_f32p), B.ctypes.data_as(_f32p),
+                                                            C.ctypes.data_as(_f32p), M, N, K, M1, M2, N1, N2, K1, number)
                 flops = (2 * M * N * K * 1e-9) / cost
                 if flops > peak_gflops * keep:
                     if (M, N, K) in cache_block_dict:
@@ -324,3 +339,37 @@ def x86_time_gemm(prof_dict, M, N, K, num_thread=None, number=100, A=None, B=Non
         raise RuntimeError("oracle_x86_time_sch_gemm failed")
     gflops = 2 * Mp * Np * Kp / 1e9 / cost
     return cost, gflops, (Mp, Np, Kp), tiling, C[:M, :N]
+
+
+def x86_changed_profile(peak_gflops=X86_PEAK_GFLOPS, number=1000, time_fn=None, keep=0.6):
+    """changed_profile_x86_CPU.py:62-127 (profile_Helix_x86_CPU_gemm_kernel of that file)."""
+    return x86_profile(peak_gflops=peak_gflops, number=number, time_fn=time_fn, keep=keep, timed_cache_blocks=True)
+
+
+def x86_conv_gemm_extents(batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
+    """The GEMM a convolution is timed as (benchmark_x86_CPU_conv.py:123-125)."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    return M, output_channel, input_channel * kH * kW
+
+
+def x86_time_conv(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, num_thread=None,
+                  number=100):
+    """get_Helix_result of benchmark_x86_CPU_conv.py:119-140: the convolution is timed as the GEMM of its
+    im2col extents on random matrices (no gather is run); returns what x86_time_gemm returns, GFLOP/s on the
+    padded extents as there (:138)."""
+    M, N, K = x86_conv_gemm_extents(batch, input_channel, H, W, output_channel, kH, kW, stride, pad)
+    return x86_time_gemm(prof_dict, M, N, K, num_thread=num_thread, number=number)
+
+
+def x86_time_model(prof_dict, mnk_list, num_thread=None, number=100):
+    """Model-level cost (benchmark_x86_CPU_model_level_LLM.py:180-195): get_Helix_result (:119-135) returns the
+    mean seconds of one GEMM and the benchmark adds them over the model's (M, N, K) list, repeats included (the
+    reference prints that sum of seconds with an "ms" label; the value is restated, not the label).  Each
+    distinct shape is timed once here and weighted by its multiplicity.  Returns total seconds."""
+    counts = {}
+    for mnk in mnk_list:
+        counts[tuple(mnk)] = counts.get(tuple(mnk), 0) + 1
+    total = 0.0
+    for (M, N, K), count in counts.items():
+        total += x86_time_gemm(prof_dict, M, N, K, num_thread=num_thread, number=number)[0] * count
+    return total

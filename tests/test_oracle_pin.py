@@ -330,6 +330,71 @@ def test_x86_profile_with_injected_clock():
     assert max(k[0] for k in cache) <= 256 and max(k[1] for k in cache) <= 256
 
 
+def test_x86_changed_profile_times_every_cache_block():
+    # changed_profile_x86_CPU.py:101-127: each cache block is run with its register block's schedule and its own
+    # extents.  A clock that charges 100 GFLOP/s to blocks narrower than 128 columns and 200 GFLOP/s from there
+    # shows that the cache blocks are timed on their own (M, N, K) -- an extrapolated cost could not depend on N --
+    # and that the register block's parameters are passed through.
+    seen = []
+
+    def clock(M, N, K, m1, m2, n1, n2, k1):
+        seen.append((M, N, K, m1, m2, n1, n2, k1))
+        return 2 * M * N * K * 1e-9 / (200.0 if N >= 128 else 100.0)
+
+    reg, cache = O.x86_changed_profile(peak_gflops=153, time_fn=clock)
+    assert len(reg) == 270                      # every register block runs at 100 > 0.6 * 153
+    assert abs(cache[(8, 96, 32)][2] - 100.0) < 1e-9 and abs(cache[(8, 128, 32)][2] - 200.0) < 1e-9
+    # the 48- and 80-wide register blocks are run as n1 = 16, n2 = 3 / 5 (changed_profile_x86_CPU.py:96-98)
+    assert (2 * 4, 48 * 2, 16 * 3, 4, 1, 16, 3, 3) in seen and (9, 80, 16, 9, 1, 16, 5, 1) in seen
+    # a cache block is K = 16 * K1 deep, a multiple of its register block in M and N, at most 256 x 256
+    for (M, N, K), (key, cost, flops) in cache.items():
+        assert M % key[0] == 0 and N % key[1] == 0 and K == 16 * key[2] and M <= 256 and N <= 256
+    # where two register blocks give the same cache block, the cheaper one is kept (:121-125)
+    def clock2(M, N, K, m1, m2, n1, n2, k1):
+        return 2 * M * N * K * 1e-9 / (100.0 + m1)
+    _, cache2 = O.x86_changed_profile(peak_gflops=153, time_fn=clock2)
+    assert cache2[(8, 16, 16)][0] == (8, 16, 1)    # reachable from M1 = 1, 2, 4, 8: the fastest clock is M1 = 8
+
+
+def test_x86_changed_profile_runs_the_real_kernel_on_cache_blocks():
+    # without an injected clock the cache blocks go through the same timed kernel as the register blocks; keep the
+    # run short: one repetition, and a peak so high that only the calibration path is exercised
+    reg, cache = O.x86_changed_profile(peak_gflops=1e9, number=1)
+    assert reg == {} and cache == {}
+
+
+def test_x86_conv_is_timed_as_the_gemm_of_its_im2col_extents():
+    # benchmark_x86_CPU_conv.py:123-125, checked on layers whose extents are known: ResNet-50 conv1 (7x7 s2 p3 on
+    # 224^2 -> 112^2), a 3x3 s1 p1 layer (same size out), a 1x1 s2 layer (56 -> 28)
+    assert O.x86_conv_gemm_extents(1, 3, 224, 224, 64, 7, 7, 2, 3) == (112 * 112, 64, 147)
+    assert O.x86_conv_gemm_extents(32, 64, 56, 56, 64, 3, 3, 1, 1) == (32 * 56 * 56, 64, 576)
+    assert O.x86_conv_gemm_extents(32, 256, 56, 56, 512, 1, 1, 2, 0) == (32 * 28 * 28, 512, 256)
+    # and equals the extents of the NHWC convolution the oracle computes
+    x = np.zeros((2, 9, 11, 4), np.float32)
+    w = np.zeros((6, 3, 2, 4), np.float32)
+    y = O.conv2d_nhwc(x, w, 2, 1)
+    M, N, K = O.x86_conv_gemm_extents(2, 4, 9, 11, 6, 3, 2, 2, 1)
+    assert (M, N, K) == (y.shape[0] * y.shape[1] * y.shape[2], y.shape[3], w[0].size)
+    prof = {(64, 64, 32): ((4, 16, 2), 1.0, 100.0)}
+    cost, gflops, padded, tiling, _ = O.x86_time_conv(prof, 1, 8, 10, 10, 24, 3, 3, 1, 1, num_thread=2, number=1)
+    assert padded == (128, 64, 72) and tiling == (4, 1, 16, 16, 1, 4, 2)       # M = 100 -> 128, N = 24 -> 64, K = 72
+    assert abs(gflops - 2 * 128 * 64 * 72 / 1e9 / cost) < 1e-6 * gflops          # GFLOP/s on the padded extents (:138)
+
+
+def test_x86_model_cost_is_the_sum_over_the_list_with_repeats(monkeypatch):
+    # benchmark_x86_CPU_model_level_LLM.py:187-193: one get_Helix_result per list entry, added up
+    calls = []
+
+    def fake(prof, M, N, K, num_thread=None, number=100, A=None, B=None):
+        calls.append((M, N, K))
+        return (M * 1e-3 + N * 1e-6, 0.0, (M, N, K), (), None)
+
+    monkeypatch.setattr(O, "x86_time_gemm", fake)
+    total = O.x86_time_model({}, [(2, 3, 4), (5, 6, 7), (2, 3, 4)])
+    assert abs(total - (2 * (2e-3 + 3e-6) + (5e-3 + 6e-6))) < 1e-12
+    assert sorted(calls) == [(2, 3, 4), (5, 6, 7)]
+
+
 def test_x86_get_tiling_hand_cases():
     # two cache blocks; cost = t * ceil(M/Mc) * ceil(ceil(N/Nc)/threads) (benchmark_x86_CPU_gemm.py:52-54)
     prof = {(64, 64, 32): ((4, 16, 2), 1.0, 100.0), (128, 96, 48): ((8, 48, 3), 2.5, 110.0)}
