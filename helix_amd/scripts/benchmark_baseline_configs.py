@@ -49,21 +49,37 @@ class Backend:
         return k[0] if self.fp32 else k[1]
 
 
+def steady_gemm(be, key, M, N, K):
+    """(ms, TFLOP/s) of configuration `key`, timed the same way for every column of a row: three repetitions of
+    10 warm-up + 10 timed launches, the fastest mean.  A single short measurement right behind a smaller problem
+    runs while the engine clock is still ramping (a cost-model pick timed that way read 15 % slower than the same
+    library a few seconds later), and the search's own minimum over hundreds of short timings is biased low."""
+    t = min(be.gemm.run_config(key, M, N, K, warmup=10, iters=10) for _ in range(3))
+    return t * 1e3, 2.0 * M * N * K / t / 1e12
+
+
+def steady_vendor(be, M, N, K):
+    lib = load(be.build.kernel_library("rocblas_f32" if be.fp32 else "rocblas_f16"))
+    mn, _, _ = lib.bench(M, N, K, warmup=10, iters=10, outer=3, rotate_bytes=0)
+    return mn * 1e3, 2.0 * M * N * K / mn / 1e12
+
+
 def square_rows(be, prof_dict, oracle=False, vendor=False):
     """Per size: the cost model's pick (Default); oracle=True adds the exhaustive per-shape search, vendor=True
     rocBLAS on the same operand layouts."""
     rows = []
     for s in S.BASELINE_SQUARE_SIZES:
         key = be.gemm.cost_model(prof_dict, s, s, s)
-        ms, tflops = be.gemm_result(prof_dict, s, s, s)
+        ms, tflops = steady_gemm(be, key, s, s, s)
         row = {"M": s, "N": s, "K": s, "config": list(key), "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
         if oracle:
-            oms, otf, okey = be.gemm_oracle(prof_dict, s, s, s)
+            _, _, okey = be.gemm_oracle(prof_dict, s, s, s)
+            oms, otf = steady_gemm(be, okey, s, s, s)
             row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2),
                         "oracle_frac_mfma_peak": round(otf * 1e12 / be.peak, 4)})
         if vendor:
-            vms, vtf = be.gemm_vendor(s, s, s)
+            vms, vtf = steady_vendor(be, s, s, s)
             row.update({"rocblas_us": round(vms * 1e3, 2), "rocblas_TFLOP/s": round(vtf, 2)})
         rows.append(row)
     return rows
@@ -144,17 +160,19 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
     total_flops = 0.0
     for (M, N, K) in S.get_baseline_bert_MNKList():
         if (M, N, K) not in memo:
-            ms, tflops = be.gemm_result(prof_dict, M, N, K)
-            row = {"M": M, "N": N, "K": K, "config": list(be.gemm.cost_model(prof_dict, M, N, K)),
+            dkey = be.gemm.cost_model(prof_dict, M, N, K)
+            ms, tflops = steady_gemm(be, dkey, M, N, K)
+            row = {"M": M, "N": N, "K": K, "config": list(dkey),
                    "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                    "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
             times = {"default": ms}
             if oracle:
-                oms, otf, okey = be.gemm_oracle(prof_dict, M, N, K)
+                _, _, okey = be.gemm_oracle(prof_dict, M, N, K)
+                oms, otf = steady_gemm(be, okey, M, N, K)
                 row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2)})
                 times["oracle"] = oms
             if vendor:
-                vms, vtf = be.gemm_vendor(M, N, K)
+                vms, vtf = steady_vendor(be, M, N, K)
                 row.update({"rocblas_us": round(vms * 1e3, 2), "rocblas_TFLOP/s": round(vtf, 2)})
                 times["rocblas"] = vms
             memo[(M, N, K)] = times
