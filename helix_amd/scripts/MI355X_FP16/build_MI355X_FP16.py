@@ -8,9 +8,9 @@ names modulo the backend tag.  Differences that follow from the target:
     an executable; the convolution path lives in the same library as the GEMM of each configuration
     (implicit GEMM), so there is no im2col artifact;
   * wave tiles are multiples of 32 rows x 16 columns of the 16x16x32 MFMA tile, K_STAGE becomes K_STAGES (the
-    pipeline holds the K tile being multiplied in LDS and one more on its way through registers: 2 is the
-    only depth the gfx950 template implements), and BLOCK_K is a template parameter too (it is fixed to 32
-    in the reference, gemm.cu:77);
+    pipeline holds the K tile being multiplied in LDS and K_STAGES - 1 more on their way through staging
+    registers: 2, and 3 for the tiles whose registers allow a second staging set), and BLOCK_K is a template
+    parameter too (it is fixed to 32 in the reference, gemm.cu:77);
   * the deeper pipelines of the reference (K_STAGE 3 .. 5 are rings of cp.async stages, gemm.cu:156-198) are the
     direct-to-LDS family, src_template/MI355X_FP16/gemm_dtl.hip: eight-wave tiles whose K tiles go from global
     memory straight into a ring of K_STAGES LDS stages of BLOCK_K = 32 or 64 columns.  Its prof-dict keys carry a
@@ -24,7 +24,7 @@ from utils.helix_runtime import SRC_ROOT, bin_dir, compile_many
 
 root_path = os.getcwd()
 
-K_STAGES_LIST = [2]
+K_STAGES_LIST = [2, 3]
 SPLITK_MAX = 8              # a split-K library partitions K 2 .. 8 ways, chosen per problem
 SPLITK_STAGES_LIST = [2]    # pipeline depths a split-K variant is built for
 WAVE_TILE_LIST = [32, 64, 128]              # wave-tile rows (the epilogue pairs 16-row MFMA tiles)
@@ -42,15 +42,18 @@ LDS_LIMIT = 160 * 1024
 VGPR_FILE = 512             # registers per lane of one SIMD (arch + accumulation), shared by its resident waves
 
 
-def vgpr_estimate(block_rows, block_cols, wave_rows, wave_cols, block_k):
+STAGES3_VGPR_MARGIN = 56     # three stages, two waves per SIMD: registers the compiler needs beyond the estimate
+STAGES3_NONACC_LIMIT = 200    # three stages, one wave per SIMD: fragments + staging + addresses in the architectural half
+
+def vgpr_estimate(block_rows, block_cols, wave_rows, wave_cols, block_k, k_stages=2):
     """Registers per lane the kernel keeps live in its main loop: FP32 accumulators, the double-buffered
     fragments of the operand with more 16-row fragments, the 4-deep window of the other one, the staging
-    registers of one K tile, and about 16 for addresses."""
+    registers of K_STAGES - 1 K tiles, and about 16 for addresses."""
     threads = 64 * (block_rows // wave_rows) * (block_cols // wave_cols)
     tm, tn = wave_rows // 16, wave_cols // 16
     acc = wave_rows * wave_cols // 64
     frags = 2 * max(tm, tn) * 4 + 4 * 4
-    staging = (block_rows + block_cols) * (block_k // 8) // threads * 4
+    staging = (block_rows + block_cols) * (block_k // 8) // threads * 4 * (k_stages - 1)
     return acc + frags + staging + 16
 
 
@@ -66,7 +69,7 @@ def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, 
     if block_cols == block_rows * 16 or block_rows == block_cols * 16:
         return False
     # gfx950 resources: two LDS stages, even split of the tile copy over threads, registers
-    if k_stages != 2:
+    if k_stages not in (2, 3):
         return False
     if 2 * (block_rows + block_cols) * block_k * 2 > LDS_LIMIT:
         return False
@@ -82,9 +85,16 @@ def is_valid_config(block_rows_scale, block_cols_scale, block_rows, block_cols, 
     if ((block_k // 32) * streamed) % (2 * min(streamed, 2)):
         return False
     waves_per_simd = (threads // 64 + 3) // 4
-    if vgpr_estimate(block_rows, block_cols, wave_rows, wave_cols, block_k) > VGPR_FILE // waves_per_simd:
-        return False
-    return True
+    estimate = vgpr_estimate(block_rows, block_cols, wave_rows, wave_cols, block_k, k_stages)
+    if k_stages == 2:
+        return estimate <= VGPR_FILE // waves_per_simd
+    # Three stages: the loop is unrolled over both staging sets and the compiler needs more than the estimate.  With
+    # one wave per SIMD the accumulators can live in the accumulation half of the file, but everything else has
+    # to fit the architectural half; with two waves per SIMD everything shares 256 registers.  (The limits are what
+    # separates the configurations that compile without scratch from those that spill.)
+    if waves_per_simd == 1:
+        return estimate - wave_rows * wave_cols // 64 <= STAGES3_NONACC_LIMIT
+    return estimate + STAGES3_VGPR_MARGIN <= VGPR_FILE // waves_per_simd
 
 
 def iter_configs():

@@ -14,8 +14,10 @@
 //   BLOCK_ROWS x BLOCK_COLS   workgroup tile of C           (reference BLOCK_ROWS / BLOCK_COLS)
 //   WAVE_ROWS  x WAVE_COLS    tile of C owned by one wave64 (reference WARP_ROWS / WARP_COLS)
 //   BLOCK_K                   K extent of one LDS stage (64 or 128)
-//   K_STAGES                  K tiles in the pipeline beside the one being loaded: the tile being multiplied
-//                             and the one on its way to LDS; 2 is the only depth    (reference K_STAGE)
+//   K_STAGES                  K tiles in the pipeline: the tile being multiplied from LDS and K_STAGES - 1 tiles on
+//                             their way through staging registers (2: one register set; 3: two, so that a load
+//                             has two tiles to land -- a few percent on mid-size tiles, where the registers allow
+//                             it)                                                  (reference K_STAGE)
 //   SPLIT_K                   1: each workgroup walks all of K.  > 1: K is partitioned over blockIdx.y into
 //                             2 .. SPLIT_K ranges, as many as it takes to give every compute unit a
 //                             workgroup (FP32 workspace + fixed-order reduction kernel)
@@ -26,7 +28,7 @@
 //     chip runs against its power limit, MFMA-only loops measure 1.95 PFLOP/s with it against 1.69.
 //   * global -> registers (128-bit buffer loads; hardware bounds checking zero-fills rows beyond M / N and
 //     the K tail) -> LDS (ds_write_b128) -> fragments (ds_read_b128).  Two LDS stages; the loads of a tile
-//     are issued one tile ahead of its LDS writes and every memory instruction sits behind its own MFMA, evenly
+//     are issued K_STAGES - 1 tiles ahead of its LDS writes and every memory instruction sits behind its own MFMA, evenly
 //     spread over the tile, so that the four waves of a workgroup never queue bursts on the CU's single
 //     address unit (a burst of 64 KiB behind a barrier costs more than the k-step it hides in).
 //   * LDS rows are BLOCK_K halves; 16-byte chunk c of row r is stored at chunk (c ^ key(r)), with
@@ -52,7 +54,8 @@ constexpr int LDS_BYTES = RING_BYTES > NWAVES * STRIP_BYTES ? RING_BYTES : NWAVE
 static_assert(BK == 64 || BK == 128, "BLOCK_K holds an even number of 32-wide MFMA k-steps: 64 or 128");
 static_assert(NTHREADS % KCH == 0, "bad thread count");
 static_assert((BM * KCH) % NTHREADS == 0 && (BN * KCH) % NTHREADS == 0, "tile copy must divide evenly");
-static_assert(STAGES == 2, "K_STAGES: one K tile staged in registers behind the one in LDS");
+static_assert(STAGES >= 2 && STAGES <= 4, "K_STAGES: one to three K tiles staged in registers behind the one in LDS");
+constexpr int RT = STAGES - 1;                 // K tiles in flight in staging registers
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
 
 __device__ __forceinline__ int swz_key(int row) { return (row / RP) & (KCH - 1); }
@@ -334,7 +337,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     // always has the next MFMA queued while the memory instructions issue in its shadow.
     constexpr Schedule sched = make_schedule();
     half8 fr[2][T_RES], fs[AW];
-    intx4 st[NV];
+    intx4 st[RT][NV];
 
     auto read_res = [&](const unsigned char* sb, int s, int v) -> half8 {
         return RES_A ? read_a(sb, s, v) : read_b(sb, s, v);
@@ -349,21 +352,24 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     auto tile_k0 = [&](int t) -> int { return t == 0 ? k_begin : k_begin + first_w + (t - 1) * BK; };
 
     if (ktiles > 0) {
-        // prologue: tile 0 into the staging registers and on to LDS, the registers refilled with tile 1
-        {
-            const __amdgpu_buffer_rsrc_t ra = rsrc_a(k_begin, true), rb = rsrc_b(k_begin, true);
+        // prologue: tiles 0 .. RT-1 into the staging register sets (tile j in set j), tile 0 on to LDS and its set
+        // refilled with tile RT
+#pragma unroll
+        for (int j = 0; j < RT; j++) {
+            const int k0 = tile_k0(j);
+            const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0, j < ktiles), rb = rsrc_b(k0, j < ktiles);
             const ConvTile ct = conv_next();
 #pragma unroll
-            for (int idx = 0; idx < NV; idx++) st[idx] = load_slot(idx, k_begin, true, first_w, ra, rb, ct);
+            for (int idx = 0; idx < NV; idx++) st[j][idx] = load_slot(idx, k0, j == 0, j == 0 ? first_w : BK, ra, rb, ct);
         }
         {
-            const int k0 = tile_k0(1);
-            const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0, 1 < ktiles), rb = rsrc_b(k0, 1 < ktiles);
+            const int k0 = tile_k0(RT);
+            const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0, RT < ktiles), rb = rsrc_b(k0, RT < ktiles);
             const ConvTile ct = conv_next();
 #pragma unroll
             for (int idx = 0; idx < NV; idx++) {
-                store_slot(idx, 0, st[idx]);
-                st[idx] = load_slot(idx, k0, false, BK, ra, rb, ct);
+                store_slot(idx, 0, st[0][idx]);
+                st[0][idx] = load_slot(idx, k0, false, BK, ra, rb, ct);
             }
         }
         __syncthreads();
@@ -381,10 +387,10 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
         }
     }
 
-    // Slots [LO, HI) of K tile kt, multiplied from LDS stage `stage`.
-    // k0c, ra, rb, ctc: start, descriptors and conv state of tile kt + 2, the one loaded into the staging
+    // Slots [LO, HI) of K tile kt, multiplied from LDS stage `stage`.  stv: the staging registers that hold tile
+    // kt + 1.  k0c, ra, rb, ctc: start, descriptors and conv state of tile kt + 1 + RT, the one loaded into those
     // registers once they are written.
-    auto tile_part = [&](auto lo_c, auto hi_c, int stage, int k0c, __amdgpu_buffer_rsrc_t ra,
+    auto tile_part = [&](auto lo_c, auto hi_c, int stage, intx4 (&stv)[NV], int k0c, __amdgpu_buffer_rsrc_t ra,
                          __amdgpu_buffer_rsrc_t rb, ConvTile ctc) {
         constexpr int LO = decltype(lo_c)::value, HI = decltype(hi_c)::value;
         const unsigned char* sb = smem + stage * STAGE_BYTES;
@@ -414,8 +420,8 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             // LDS writes of the staged tile and the refills of their registers
 #pragma unroll
             for (int idx = 0; idx < NV; idx++) {
-                if (sched.wslot[idx] == g) store_slot(idx, stage ^ 1, st[idx]);
-                if (sched.lslot[idx] == g) st[idx] = load_slot(idx, k0c, false, BK, ra, rb, ctc);
+                if (sched.wslot[idx] == g) store_slot(idx, stage ^ 1, stv[idx]);
+                if (sched.lslot[idx] == g) stv[idx] = load_slot(idx, k0c, false, BK, ra, rb, ctc);
             }
             __builtin_amdgcn_sched_barrier(0);
           }
@@ -424,19 +430,40 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     constexpr std::integral_constant<int, 0> c_0{};
     constexpr std::integral_constant<int, G_BAR> c_bar{};
     constexpr std::integral_constant<int, G> c_end{};
-    int stage = 0;
-    for (int kt = 0; kt < ktiles; kt++) {
-        const int kt_ld = kt + 2;
+    // one K tile: multiply tile kt from `stage`, move tile kt + 1 from its registers to the other stage, refill them
+    // with tile kt + 1 + RT
+    auto tile_step = [&](int kt, int stage, intx4 (&stv)[NV]) {
+        const int kt_ld = kt + 1 + RT;
         const int k0c = tile_k0(kt_ld);
         // past the last tile the loads still issue, with empty descriptors, which keeps the body branch-free
         const __amdgpu_buffer_rsrc_t ra = rsrc_a(k0c, kt_ld < ktiles), rb = rsrc_b(k0c, kt_ld < ktiles);
         const ConvTile ctc = conv_next();
-        tile_part(c_0, c_bar, stage, k0c, ra, rb, ctc);
+        tile_part(c_0, c_bar, stage, stv, k0c, ra, rb, ctc);
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         __builtin_amdgcn_sched_barrier(0);
-        tile_part(c_bar, c_end, stage, k0c, ra, rb, ctc);
-        stage ^= 1;
+        tile_part(c_bar, c_end, stage, stv, k0c, ra, rb, ctc);
+    };
+    // tile kt + 1 sits in register set (kt + 1) % RT and LDS stage (kt + 1) % 2.  One register set: a plain loop
+    // with the stage as a variable (unrolling it doubles the register pressure of the one-wave tiles, whose copy
+    // slots already fill the file).  More sets: the loop is unrolled over the least common multiple of the two
+    // periods so that the set is a compile-time constant.
+    constexpr int UNROLL = (RT % 2 == 0) ? RT : 2 * RT;
+    if constexpr (RT == 1) {
+        int stage = 0;
+        for (int kt = 0; kt < ktiles; kt++) {
+            tile_step(kt, stage, st[0]);
+            stage ^= 1;
+        }
+    } else {
+        int kt = 0;
+        for (; kt + UNROLL <= ktiles; kt += UNROLL) {
+#pragma unroll
+            for (int u = 0; u < UNROLL; u++) tile_step(kt + u, u & 1, st[(u + 1) % RT]);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL - 1; u++)
+            if (kt + u < ktiles) tile_step(kt + u, u & 1, st[(u + 1) % RT]);
     }
 
     store_tile(acc, p, m0, n0, wave, wave_m, wave_n, lane, smem);

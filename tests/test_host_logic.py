@@ -24,7 +24,8 @@ from MI355X_FP32 import MI355X_FP32_conv as c32
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 N_FP16_CONFIGS = 159   # points of the FP16 template space (tile x wave tile x BLOCK_K) that fit LDS and registers
-N_FP16_SPLITK = 159    # every point also has a split-K variant
+N_FP16_STAGES3 = 86    # of those, the points whose registers also hold a second staging set (K_STAGES = 3)
+N_FP16_SPLITK = 159    # every two-stage point also has a split-K variant
 N_FP16_DTL = 68        # points of the direct-to-LDS family: eight-wave tiles x (BLOCK_K, K_STAGES) in {32: 3, 4; 64: 2, 3}
 
 
@@ -38,24 +39,35 @@ def test_fp16_reference_validity_rules():
     assert b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 2)
     # gfx950 resource rules
     assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 128, 2)  # 2 x 512 x 128 x 2 B > 160 KiB of LDS
-    assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 3)   # only the two-tile pipeline exists
+    assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 3)   # no registers for a second staging set
+    assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 4)   # two or three stages only
+    assert b16.is_valid_config(2, 2, 128, 128, 64, 64, 64, 3)         # four waves, 64 accumulator registers each
     assert b16.is_valid_config(2, 4, 256, 256, 128, 64, 64, 2)        # 8 waves x 256 registers
     assert b16.vgpr_estimate(256, 256, 128, 128, 64) == 256 + 80 + 64 + 16
     assert b16.vgpr_estimate(256, 256, 128, 64, 64) == 128 + 80 + 32 + 16      # exactly the 256 of two waves per SIMD
+    assert b16.vgpr_estimate(128, 128, 64, 64, 64, 3) == 64 + 48 + 2 * 32 + 16   # two staging sets
 
 
 def test_fp16_template_space():
     cfgs = list(b16.iter_configs())
-    assert len(cfgs) == N_FP16_CONFIGS and len(set(cfgs)) == N_FP16_CONFIGS
+    assert len(cfgs) == N_FP16_CONFIGS + N_FP16_STAGES3 and len(set(cfgs)) == len(cfgs)
+    assert sum(1 for c in cfgs if c[0] == 2) == N_FP16_CONFIGS
     for (st, br, bc, wr, wc, bk) in cfgs:
         assert br % wr == 0 and bc % wc == 0 and br <= 256 and bc <= 256
-        assert st == 2 and bk in (64, 128) and 2 * (br + bc) * bk * 2 <= 160 * 1024
+        assert st in (2, 3) and bk in (64, 128) and 2 * (br + bc) * bk * 2 <= 160 * 1024
         threads = 64 * (br // wr) * (bc // wc)
         assert threads <= 512 and (br * bk // 8) % threads == 0 and (bc * bk // 8) % threads == 0
-        assert b16.vgpr_estimate(br, bc, wr, wc, bk) <= 512 // ((threads // 64 + 3) // 4)
-    assert (2, 256, 256, 128, 128, 64) in cfgs
+        assert b16.vgpr_estimate(br, bc, wr, wc, bk, st) <= 512 // ((threads // 64 + 3) // 4)
+        if st == 3:      # every three-stage point is a two-stage point with room for the second staging set
+            assert (2, br, bc, wr, wc, bk) in cfgs
+    assert (2, 256, 256, 128, 128, 64) in cfgs and (3, 256, 128, 64, 64, 64) in cfgs
+    assert (3, 256, 256, 64, 128, 64) not in cfgs and (3, 256, 192, 64, 96, 64) not in cfgs
     keys = p16.all_keys()
-    assert len(keys) == N_FP16_CONFIGS + N_FP16_SPLITK + N_FP16_DTL + 6
+    # a three-stage point whose GEMM kernel was recorded as spilling at build time is left out of the key list
+    spilling3 = sum(1 for (st, br, bc, wr, wc, bk) in cfgs
+                    if st == 3 and p16.gemm_kernel_scratch((st, br, bc, wr, wc, 0, bk)) > 0)
+    assert len(keys) == N_FP16_CONFIGS + N_FP16_STAGES3 - spilling3 + N_FP16_SPLITK + N_FP16_DTL + 6
+    assert not any(k[0] == 3 and k[5] == 1 and not b16.is_dtl_key(k) for k in keys)    # split-K is built for two stages
     # seven fields; the direct-to-LDS family carries a trailing eighth field 1
     assert all(len(k) == (8 if b16.is_dtl_key(k) else 7) for k in keys)
     assert sum(1 for k in keys if b16.is_dtl_key(k)) == N_FP16_DTL
