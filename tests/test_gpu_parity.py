@@ -227,6 +227,24 @@ def test_gemv_f16_integer_inputs_exact():
             want = x.astype(np.int64) @ W.astype(np.int64)
             assert np.abs(want).max() < 2048
             assert np.array_equal(run_gemm_f16(lib, x, W).astype(np.int64), want), (name, M, N, K)
+            # leading dimensions wider than K (rows 16 bytes apart from the packed layout)
+            assert np.array_equal(run_gemm_f16(lib, x, W, ldpad=8).astype(np.int64), want), (name, M, N, K, "ld")
+
+
+def test_gemv_f16_streamed_mfma_work_splits():
+    """The two work splits of the LDS-streamed MFMA variant (9 or more activation rows): few weight rows and a long K
+    (the waves of a workgroup split the columns and add their sums through LDS), many rows (a wave owns its row
+    groups), with K ranges over grid z on top, ragged in every extent; integer-valued, so exact in any order."""
+    rng = np.random.default_rng(66)
+    for name in ("gemv", "gemv_splitK"):
+        lib = load(b16.kernel_library(name))
+        for (M, N, K) in [(16, 48, 8192), (9, 17, 5000), (13, 4096, 4096), (16, 30000, 264), (10, 130, 1032),
+                          (16, 2000, 3080), (33, 64, 2048)]:
+            x = rng.integers(-1, 2, (M, K)).astype(np.float16)
+            W = rng.integers(-1, 2, (K, N)).astype(np.float16)
+            want = x.astype(np.int64) @ W.astype(np.int64)
+            assert np.abs(want).max() < 2048
+            assert np.array_equal(run_gemm_f16(lib, x, W).astype(np.int64), want), (name, M, N, K)
 
 
 def test_gemv_f16_baseline_shapes_sampled():
