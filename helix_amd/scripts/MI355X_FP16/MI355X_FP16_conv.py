@@ -30,8 +30,31 @@ GENERAL_GATHER_COST_PER_64_K = 0.3
 GENERAL_GATHER_COST_PER_128_ROWS = 0.2
 
 
+# A layer of few K tiles (1x1 layers, first layers) is mostly first loads and result stores around a short multiply.
+# Workgroups that share a compute unit overlap those phases, a workgroup that fills the unit alone runs them one
+# after the other: over such layers the measured time follows 1 + this / (workgroups resident per compute unit),
+# and the gather term per tile column is half as large.
+SHORT_K_TILES = 8
+SHORT_K_ALONE_COST = 0.6
+SHORT_K_GATHER_COST_PER_TILE_COLUMN = 0.1
+LDS_BYTES_PER_CU = 160 * 1024
+WAVES_PER_CU = 16
+
+
+def resident_workgroups(k):
+    """Workgroups of configuration k that fit one compute unit: two LDS stages of (rows + columns) x BLOCK_K halves
+    each, at most 16 waves, at most 8 workgroups."""
+    lds = 2 * (k[1] + k[2]) * k[6] * 2
+    waves = (k[1] // k[3]) * (k[2] // k[4])
+    return max(1, min(LDS_BYTES_PER_CU // lds, WAVES_PER_CU // waves, 8))
+
+
 def conv_config_cost(k, v, M, N, K, v_short=None, IC=None):
-    cost = config_cost(k, v, M, N, K, v_short) * (1.0 + GATHER_COST_PER_TILE_COLUMN * math.ceil(N / k[2]))
+    short = math.ceil(K / k[6]) <= SHORT_K_TILES
+    per_column = SHORT_K_GATHER_COST_PER_TILE_COLUMN if short else GATHER_COST_PER_TILE_COLUMN
+    cost = config_cost(k, v, M, N, K, v_short) * (1.0 + per_column * math.ceil(N / k[2]))
+    if short:
+        cost *= 1.0 + SHORT_K_ALONE_COST / resident_workgroups(k)
     if IC is not None and IC % k[6]:
         cost *= (1.0 + GENERAL_GATHER_COST_PER_64_K * k[6] / 64) * (1.0 + GENERAL_GATHER_COST_PER_128_ROWS * k[1] / 128)
     return cost

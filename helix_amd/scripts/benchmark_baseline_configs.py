@@ -58,6 +58,18 @@ def steady_gemm(be, key, M, N, K):
     return t * 1e3, 2.0 * M * N * K / t / 1e12
 
 
+def steady_oracle(be, prof_dict, dkey, dms, M, N, K):
+    """(ms, TFLOP/s, key) of the exhaustive search's pick, timed like the Default column.  The Default configuration
+    is one of the candidates, so when the search returns it again, or a configuration that the steadier timing shows
+    to be slower, the row's Oracle column is the Default measurement itself."""
+    _, _, okey = be.gemm_oracle(prof_dict, M, N, K)
+    if tuple(okey) != tuple(dkey):
+        oms, otf = steady_gemm(be, okey, M, N, K)
+        if oms < dms:
+            return oms, otf, okey
+    return dms, 2.0 * M * N * K / (dms * 1e-3) / 1e12, dkey
+
+
 def steady_vendor(be, M, N, K):
     lib = load(be.build.kernel_library("rocblas_f32" if be.fp32 else "rocblas_f16"))
     mn, _, _ = lib.bench(M, N, K, warmup=10, iters=10, outer=3, rotate_bytes=0)
@@ -74,8 +86,7 @@ def square_rows(be, prof_dict, oracle=False, vendor=False):
         row = {"M": s, "N": s, "K": s, "config": list(key), "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
         if oracle:
-            _, _, okey = be.gemm_oracle(prof_dict, s, s, s)
-            oms, otf = steady_gemm(be, okey, s, s, s)
+            oms, otf, okey = steady_oracle(be, prof_dict, key, ms, s, s, s)
             row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2),
                         "oracle_frac_mfma_peak": round(otf * 1e12 / be.peak, 4)})
         if vendor:
@@ -143,6 +154,8 @@ def conv_rows(be, prof_dict, vendor=False, oracle=False):
                      "frac_hbm_peak": round(nbytes / (ms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
         if conv_oracle is not None:
             oms, otf, okey = conv_oracle(prof_dict, *shp)
+            if oms >= ms:   # the Default configuration is one of the candidates
+                oms, otf, okey = ms, tflops, key
             rows[-1].update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2),
                              "oracle_frac_mfma_peak": round(otf * 1e12 / be.peak, 4),
                              "oracle_frac_hbm_peak": round(nbytes / (oms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
@@ -167,8 +180,7 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
                    "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
             times = {"default": ms}
             if oracle:
-                _, _, okey = be.gemm_oracle(prof_dict, M, N, K)
-                oms, otf = steady_gemm(be, okey, M, N, K)
+                oms, otf, okey = steady_oracle(be, prof_dict, dkey, ms, M, N, K)
                 row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2)})
                 times["oracle"] = oms
             if vendor:

@@ -218,6 +218,15 @@ def test_fp16_cost_model_two_point_profile():
     assert c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6, IC=8) == pytest.approx(
         c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6) * (1 + c16.GENERAL_GATHER_COST_PER_64_K * big[6] / 64)
         * (1 + c16.GENERAL_GATHER_COST_PER_128_ROWS * big[1] / 128))
+    # few K tiles: the gather term halves and a workgroup alone on its compute unit pays for not overlapping its phases
+    assert c16.resident_workgroups(big) == 1 and c16.resident_workgroups(small) == 6
+    assert c16.resident_workgroups((2, 128, 128, 64, 32, 0, 64)) == 2 and c16.resident_workgroups((2, 64, 64, 32, 32, 0, 64)) == 4
+    Kshort = c16.SHORT_K_TILES * big[6]
+    assert c16.conv_config_cost(big, 60e-6, 4096, 512, Kshort, 8e-6) == pytest.approx(
+        g16.config_cost(big, 60e-6, 4096, 512, Kshort, 8e-6) * (1 + 2 * c16.SHORT_K_GATHER_COST_PER_TILE_COLUMN)
+        * (1 + c16.SHORT_K_ALONE_COST / 1))
+    assert c16.conv_config_cost(big, 60e-6, 4096, 512, Kshort + big[6], 8e-6) == pytest.approx(
+        g16.config_cost(big, 60e-6, 4096, 512, Kshort + big[6], 8e-6) * (1 + 2 * c16.GATHER_COST_PER_TILE_COLUMN))
     # channel counts off the gather chunk: padded when that is at most 8/3 of the real count, else left alone
     assert [c16.gather_channels(c) for c in (1, 2, 3, 6, 8, 25, 64)] == [1, 2, 8, 8, 8, 32, 64]
     assert [c32.gather_channels(c) for c in (1, 2, 3, 6, 8, 25, 64)] == [1, 4, 4, 8, 8, 28, 64]
