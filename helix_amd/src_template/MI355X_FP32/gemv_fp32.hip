@@ -49,6 +49,9 @@
 #ifndef X_LDS_BYTES_WIDE
 #define X_LDS_BYTES_WIDE 131072   // ... of one workgroup of twice as many waves, alone on its CU: same waves per CU
 #endif
+#ifndef GEMV_MANY_WAVES_MT
+#define GEMV_MANY_WAVES_MT 2   // activation-row tiles up to this one run 16 waves per compute unit instead of 8
+#endif
 #ifndef TARGET_WAVES
 #define TARGET_WAVES 2048   // waves a launch aims for: 256 compute units x 8
 #endif
@@ -355,12 +358,17 @@ inline int launch_waves(Params p, int lds, hipStream_t s) {
 
 template <int MT, int ROWS, int KU>
 inline int launch_cfg(Params p, hipStream_t s) {
-    // consecutive rows per wave: a multiple of ROWS that brings the launch near TARGET_WAVES waves
-    long long want = ((long long)p.N * p.ksplit + TARGET_WAVES - 1) / TARGET_WAVES;
+    // One or two activation rows leave the vector units idle most of the time: twice the waves per CU, in workgroups
+    // of twice the size so that the activations are staged as often as before (measured 2 - 7 % on the decode shapes;
+    // slower from four rows on).
+    const int lds = MT * p.kchunk * 4;
+    const bool many = (MT <= GEMV_MANY_WAVES_MT) && lds <= X_LDS_BYTES;
+    const long long target = many ? 2 * TARGET_WAVES : TARGET_WAVES;
+    // consecutive rows per wave: a multiple of ROWS that brings the launch near the target number of waves
+    long long want = ((long long)p.N * p.ksplit + target - 1) / target;
     if (want < 1) want = 1;
     p.rows_per_wave = (int)((want + ROWS - 1) / ROWS) * ROWS;
-    const int lds = MT * p.kchunk * 4;
-    if (lds > X_LDS_BYTES) return launch_waves<MT, ROWS, KU, 2 * WPB>(p, lds, s);
+    if (many || lds > X_LDS_BYTES) return launch_waves<MT, ROWS, KU, 2 * WPB>(p, lds, s);
     return launch_waves<MT, ROWS, KU, WPB>(p, lds, s);
 }
 
