@@ -38,7 +38,7 @@
 //     every copy instruction (buffer_load ... lds) fetches 512 contiguous bytes of each of two rows -- whole-row
 //     spans, the pattern that streams fastest -- and the MFMA operands (lane l: row l % 16, columns 8*(l/16) .. +7 of
 //     a 32-wide block) are read back from LDS.  Loading the operand layout straight into registers (16 rows x 64
-//     bytes per instruction) measured 4.3 TB/s on 8192 x 28672 weights at 16 rows, this variant 5.3;
+//     bytes per instruction) measured 4.3 TB/s on 8192 x 28672 weights at 16 rows, this variant 5.8;
 //   * eight MFMAs per step accumulate the 16 x 16 block y[m][n]; copies run three steps ahead; buffer bounds
 //     checking zero-fills weight rows beyond N;
 //   * two work splits: a wave owns its own row groups and all columns of the K range, or the four waves of a
@@ -379,8 +379,9 @@ __device__ __forceinline__ intx4 raw_rsrc(const void* base, unsigned bytes) {
 
 // 16 bytes per lane from the buffer straight to LDS byte lds_addr + 16 * lane (out-of-range lanes store zeros).
 // Inline assembly: completion is tracked by hand with wait_vmcnt, the compiler does not count these.
+// Non-temporal: the weights are read once (measured 10 % faster than the default policy on 8192 x 28672 at 16 rows).
 __device__ __forceinline__ void dma16(intx4 rsrc, unsigned lds_addr, int voff) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds"
                  :
                  : "s"(lds_addr), "v"(voff), "s"(rsrc)
                  : "memory", "m0");
