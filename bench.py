@@ -27,7 +27,7 @@ SIZE = 8192
 MEASURED_TRAFFIC = {
     (2, 256, 256, 64, 128, 0, 64): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
     (2, 256, 256, 128, 64, 0, 64): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
-    (2, 256, 256, 128, 128, 0, 64): (1.746e9, "profiles/gemm_f16_8192_pmc.md"),
+    (2, 256, 256, 128, 128, 0, 64): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
     (2, 256, 256, 64, 128, 0, 64, 1): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
     (2, 256, 256, 128, 64, 0, 64, 1): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
 }
