@@ -13,7 +13,7 @@ import os
 
 from utils.helix_runtime import load, kernel_resources
 from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, is_dtl_key
-from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost
+from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, VERIFY_TOP
 
 root_path = os.getcwd()
 
@@ -97,6 +97,39 @@ def cost_model(prof_dict, M, N, K, IC=None):
             min_cost = cost
             best_config = k
     return best_config
+
+
+def ranked_configs(prof_dict, M, N, K, IC=None, top=VERIFY_TOP):
+    """The `top` convolution-capable configurations with the lowest predicted cost, best first; cost_model returns
+    the first of them."""
+    cand = []
+    for k, v in prof_dict.items():
+        if k[0] == 0 or is_dtl_key(k) or conv_kernel_scratch(k, IC) > 0:
+            continue
+        cand.append((conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC), k))
+    cand.sort()
+    return [k for _, k in cand[:top]]
+
+
+def get_MI355X_FP16_conv_Verified_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
+                                         top=VERIFY_TOP):
+    """The fastest of the cost model's first `top` configurations on this layer: each timed briefly, the winner timed
+    again with the runner's launch counts.  Returns (cost_ms, tflops, key)."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    flops = 2.0 * M * output_channel * input_channel * kH * kW
+    ICg = gather_channels(input_channel)
+    timed = []
+    for k in ranked_configs(prof_dict, M, output_channel, ICg * kH * kW, ICg, top):
+        try:
+            _, avg, _ = load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride,
+                                                            pad, warmup=2, iters=5)
+        except Exception:
+            continue
+        timed.append((avg, k))
+    best = min(timed)[1]
+    _, cost, _ = load(library_for_key(best)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
+                                                        warmup=10, iters=10)
+    return cost * 1e3, flops / 1e12 / cost, best
 
 
 def get_MI355X_FP16_conv_Helix_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,

@@ -1,12 +1,12 @@
 """Search-quality ablation of the MI355X_FP16 backend: exhaustive search (Oracle), the cost model
-(Default), block tile == wave tile only (Static1) and the globally fastest tile (Static2).
+(Default), the fastest of the cost model's first few candidates (Verified), block tile == wave tile only (Static1) and the globally fastest tile (Static2).
 Mirrors scripts/Ampere_FP16/benchmark_Ampere_FP16_performance_comparison.py:8-106."""
 import math
 import os
 
 from utils.get_benchmark_shape_list import get_gemm_op_MNKList
 from utils.helix_runtime import read_prof_dict
-from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, cost_model, run_config, get_MI355X_FP16_gemm_Oracle_result
+from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, cost_model, run_config, get_MI355X_FP16_gemm_Oracle_result, get_MI355X_FP16_gemm_Verified_result
 
 root_path = os.getcwd()
 
@@ -50,6 +50,10 @@ def get_Helix_Oracle_result(prof_dict, M, N, K):
     return get_MI355X_FP16_gemm_Oracle_result(prof_dict, M, N, K)[1]
 
 
+def get_Helix_Verified_result(prof_dict, M, N, K):
+    return get_MI355X_FP16_gemm_Verified_result(prof_dict, M, N, K)[1]
+
+
 def get_Helix_Static1_result(prof_dict, M, N, K):
     return _tflops(cost_model_static1(prof_dict, M, N, K), M, N, K)
 
@@ -66,6 +70,7 @@ if __name__ == "__main__":
     for M, N, K in MNKList:
         helix_oracle_flops = get_Helix_Oracle_result(prof_dict, M, N, K)
         helix_default_flops = get_Helix_Default_result(prof_dict, M, N, K)
+        helix_verified_flops = get_Helix_Verified_result(prof_dict, M, N, K)
         helix_static1_flops = get_Helix_Static1_result(prof_dict, M, N, K)
         helix_static2_flops = get_Helix_Static2_result(prof_dict, M, N, K)
-        print(f'{M}x{N}x{K}: Helix_Oracle: {helix_oracle_flops:.2f} TFlops, Helix_Default: {helix_default_flops:.2f} TFlops, Helix_Static1: {helix_static1_flops:.2f} TFlops, Helix_Static2: {helix_static2_flops:.2f} TFlops')
+        print(f'{M}x{N}x{K}: Helix_Oracle: {helix_oracle_flops:.2f} TFlops, Helix_Default: {helix_default_flops:.2f} TFlops, Helix_Verified: {helix_verified_flops:.2f} TFlops, Helix_Static1: {helix_static1_flops:.2f} TFlops, Helix_Static2: {helix_static2_flops:.2f} TFlops')

@@ -132,6 +132,17 @@ def cost_model(prof_dict, M, N, K):
     return best_config
 
 
+# "Verified" selection: the cost model ranks, the device decides among the first few (the leading predictions lie
+# within a per cent of each other for configurations that measure 5 - 10 % apart).
+VERIFY_TOP = 6
+
+
+def ranked_configs(prof_dict, M, N, K, top=VERIFY_TOP):
+    """The `top` configurations with the lowest predicted cost, best first; cost_model returns the first of them."""
+    ranked = sorted(prof_dict.items(), key=lambda kv: config_cost(kv[0], kv[1], M, N, K, extra_points(prof_dict, kv[0])))
+    return [k for k, _ in ranked[:top]]
+
+
 def run_config(k, M, N, K, warmup=10, iters=10, outer=1):
     """Seconds per launch (mean) on the real M, N, K (edges are predicated in the kernel; the reference
     pads M and N up to the tile instead, Ampere_FP32_gemm.py:103)."""
@@ -161,6 +172,20 @@ def get_MI355X_FP32_gemm_rocblas_result(M, N, K):
     _, avg, _ = lib.bench(M, N, K, warmup=10, iters=10, outer=1, rotate_bytes=0)
     cost = avg * 1e3
     return cost, 2 * M * N * K / 1e9 / cost
+
+
+def get_MI355X_FP32_gemm_Verified_result(prof_dict, M, N, K, top=VERIFY_TOP):
+    """The fastest of the cost model's first `top` configurations: each timed briefly, the winner timed again with
+    the runner's launch counts.  Returns (cost_ms, tflops, key)."""
+    timed = []
+    for k in ranked_configs(prof_dict, M, N, K, top):
+        try:
+            timed.append((run_config(k, M, N, K, warmup=2, iters=5), k))
+        except Exception:
+            continue
+    best = min(timed)[1]
+    cost = run_config(best, M, N, K)
+    return cost * 1e3, 2 * M * N * K / 1e12 / cost, best
 
 
 def get_MI355X_FP32_gemm_Oracle_result(prof_dict, M, N, K):

@@ -34,6 +34,8 @@ class Backend:
                                                          mod(f"build_{name}"), mod(f"profile_{name}"))
         self.gemm_result = getattr(self.gemm, f"get_{name}_gemm_Helix_result")
         self.gemm_oracle = getattr(self.gemm, f"get_{name}_gemm_Oracle_result")
+        self.gemm_verified = getattr(self.gemm, f"get_{name}_gemm_Verified_result")
+        self.conv_verified = getattr(self.conv, f"get_{name}_conv_Verified_result")
         self.conv_result = getattr(self.conv, f"get_{name}_conv_Helix_result")
         self.gemm_vendor = getattr(self.gemm, f"get_{name}_gemm_rocblas_result")
 
@@ -70,6 +72,17 @@ def steady_oracle(be, prof_dict, dkey, dms, M, N, K):
     return dms, 2.0 * M * N * K / (dms * 1e-3) / 1e12, dkey
 
 
+def steady_verified(be, prof_dict, dkey, dms, M, N, K):
+    """(ms, TFLOP/s, key) of Verified mode (the fastest of the cost model's first few candidates, the Default
+    configuration among them), timed like the Default column."""
+    _, _, vkey = be.gemm_verified(prof_dict, M, N, K)
+    if tuple(vkey) != tuple(dkey):
+        vms, vtf = steady_gemm(be, vkey, M, N, K)
+        if vms < dms:
+            return vms, vtf, vkey
+    return dms, 2.0 * M * N * K / (dms * 1e-3) / 1e12, dkey
+
+
 def steady_vendor(be, M, N, K):
     lib = load(be.build.kernel_library("rocblas_f32" if be.fp32 else "rocblas_f16"))
     mn, _, _ = lib.bench(M, N, K, warmup=10, iters=10, outer=3, rotate_bytes=0)
@@ -77,14 +90,16 @@ def steady_vendor(be, M, N, K):
 
 
 def square_rows(be, prof_dict, oracle=False, vendor=False):
-    """Per size: the cost model's pick (Default); oracle=True adds the exhaustive per-shape search, vendor=True
-    rocBLAS on the same operand layouts."""
+    """Per size: the cost model's pick (Default) and the fastest of its first few candidates (Verified); oracle=True
+    adds the exhaustive per-shape search, vendor=True rocBLAS on the same operand layouts."""
     rows = []
     for s in S.BASELINE_SQUARE_SIZES:
         key = be.gemm.cost_model(prof_dict, s, s, s)
         ms, tflops = steady_gemm(be, key, s, s, s)
         row = {"M": s, "N": s, "K": s, "config": list(key), "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
+        vms, vtf, vkey = steady_verified(be, prof_dict, key, ms, s, s, s)
+        row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
         if oracle:
             oms, otf, okey = steady_oracle(be, prof_dict, key, ms, s, s, s)
             row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2),
@@ -152,6 +167,10 @@ def conv_rows(be, prof_dict, vendor=False, oracle=False):
                      "TFLOP/s": round(tflops, 2), "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4),
                      "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / (ms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
+        vms, vtf, vkey = be.conv_verified(prof_dict, *shp)
+        if vms >= ms:   # the Default configuration is the first candidate
+            vms, vkey = ms, key
+        rows[-1].update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2)})
         if conv_oracle is not None:
             oms, otf, okey = conv_oracle(prof_dict, *shp)
             if oms >= ms:   # the Default configuration is one of the candidates
@@ -169,7 +188,7 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
     latency, as the reference sums per-GEMM costs (benchmark_Ampere_FP16_model_level_LLM.py:16-27).  oracle=True adds
     the exhaustive per-shape search ("per-shape autotune"), vendor=True rocBLAS."""
     memo, rows = {}, []
-    totals = {"default": 0.0, "oracle": 0.0, "rocblas": 0.0}
+    totals = {"default": 0.0, "verified": 0.0, "oracle": 0.0, "rocblas": 0.0}
     total_flops = 0.0
     for (M, N, K) in S.get_baseline_bert_MNKList():
         if (M, N, K) not in memo:
@@ -179,6 +198,9 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
                    "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                    "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
             times = {"default": ms}
+            vms, vtf, vkey = steady_verified(be, prof_dict, dkey, ms, M, N, K)
+            row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
+            times["verified"] = vms
             if oracle:
                 oms, otf, okey = steady_oracle(be, prof_dict, dkey, ms, M, N, K)
                 row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2)})
@@ -194,6 +216,8 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
         total_flops += 2.0 * M * N * K
     tf = total_flops / (totals["default"] * 1e-3) / 1e12
     total = {"total_ms": round(totals["default"], 4), "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf * 1e12 / be.peak, 4)}
+    vtf = total_flops / (totals["verified"] * 1e-3) / 1e12
+    total.update({"verified_total_ms": round(totals["verified"], 4), "verified_TFLOP/s": round(vtf, 2)})
     if oracle:
         otf = total_flops / (totals["oracle"] * 1e-3) / 1e12
         total.update({"oracle_total_ms": round(totals["oracle"], 4), "oracle_TFLOP/s": round(otf, 2),

@@ -49,6 +49,29 @@ def test_performance_comparison_default_close_to_oracle(prof16):
     assert geomean > 0.85, ratios
 
 
+def test_verified_selection_is_one_of_the_ranked_candidates_and_not_slower(prof16):
+    """Verified mode (GEMM and convolution): the returned configuration is one of the cost model's first few, the
+    first of which is the Default pick, and its time is not clearly worse than the Default pick's."""
+    from MI355X_FP16 import MI355X_FP16_gemm as g16, MI355X_FP16_conv as c16
+    for (M, N, K) in [(2048, 2048, 2048), (4096, 768, 3072), (1949, 11008, 4096)]:
+        ranked = g16.ranked_configs(prof16, M, N, K)
+        assert len(ranked) == g16.VERIFY_TOP and ranked[0] == g16.cost_model(prof16, M, N, K)
+        ms, tflops, key = g16.get_MI355X_FP16_gemm_Verified_result(prof16, M, N, K)
+        assert key in ranked and tflops > 0
+        default_ms = min(g16.run_config(ranked[0], M, N, K) for _ in range(2)) * 1e3
+        assert ms < 1.15 * default_ms, (M, N, K, key, ms, default_ms)
+    layer = (32, 64, 56, 56, 256, 1, 1, 1, 0)
+    b, ic, h, w, oc, kh, kw, st, pd = layer
+    Mc = b * ((h + 2 * pd - kh) // st + 1) * ((w + 2 * pd - kw) // st + 1)
+    ranked = c16.ranked_configs(prof16, Mc, oc, c16.gather_channels(ic) * kh * kw, c16.gather_channels(ic))
+    assert ranked[0] == c16.cost_model(prof16, Mc, oc, c16.gather_channels(ic) * kh * kw, c16.gather_channels(ic))
+    ms, tflops, key = c16.get_MI355X_FP16_conv_Verified_result(prof16, *layer)
+    assert key in ranked and tflops > 0
+    default_ms, _ = c16.get_MI355X_FP16_conv_Helix_result(prof16, *layer)
+    assert ms < 1.15 * default_ms, (key, ms, default_ms)
+    assert cmp16.get_Helix_Verified_result(prof16, 1024, 1024, 1024) > 0
+
+
 def test_adaptive_dispatch_follows_the_faster_family(prof16):
     """M = 1 .. 16 activation rows against 4096 x 1024 and 28672 x 8192 weights: the pick over all libraries is not
     clearly slower than the better of {GEMV library, best-predicted MFMA tile}."""

@@ -175,6 +175,12 @@ def test_fp16_cost_model_hand_cases():
 def test_static_cost_models():
     d = {(2, 128, 128, 64, 64, 0, 64): 1.0, (2, 64, 64, 64, 64, 0, 64): 0.4, (2, 256, 128, 64, 64, 0, 64): 1.8,
          (0, 1, 128, 0, 0, 0, 0): 1e-9}
+    # Verified mode ranks with the same costs: the Default pick first, then by predicted cost
+    ranked = g16.ranked_configs(d, 4096, 4096, 4096, top=3)
+    assert ranked[0] == g16.cost_model(d, 4096, 4096, 4096) and len(ranked) == 3
+    costs = [g16.config_cost(k, d[k], 4096, 4096, 4096, g16.short_value(d, k)) for k in ranked]
+    assert costs == sorted(costs) and max(costs) <= min(g16.config_cost(k, v, 4096, 4096, 4096, g16.short_value(d, k))
+                                                        for k, v in d.items() if k not in ranked)
     assert cmp16.cost_model_static1(d, 4096, 4096, 4096) == (2, 64, 64, 64, 64, 0, 64)     # only block == wave tile
     assert cmp16.cost_model_static2(d, 64, 64, 64) == (2, 256, 128, 64, 64, 0, 64)         # best time per tile area
 
