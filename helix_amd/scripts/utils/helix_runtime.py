@@ -45,10 +45,20 @@ def prof_dict_path(backend):
     return f"{root_path}/build/prof_dict/{backend}_cost_model.dict"
 
 
-def compile_command(src, out, defines, link=""):
-    """hipcc line of one library; `link` holds extra linker flags (the vendor comparators' -lrocblas)."""
+# The tile kernels fix their own instruction order (a scheduling fence behind every MFMA slot), but the compiler's
+# scheduler in front of the register allocator still decides the register pressure.  Where a default build leaves a
+# kernel spilling, compile_many builds the library once more with this option and keeps that build when no kernel in
+# it spills more and the sum over the kernels is smaller.
+NO_SCHEDULER_OPTION = "-mllvm -enable-misched=0"
+
+
+def compile_command(src, out, defines, link="", extra=""):
+    """hipcc line of one library; `link` holds extra linker flags (the vendor comparators' -lrocblas), `extra`
+    further compiler options."""
     inc = _find_include_dir()
     cmd = f"{HIPCC} {src} {COMPILE_OPTIONS} -I{inc} -I{os.path.join(SRC_ROOT, 'common')}"
+    if extra:
+        cmd += f" {extra}"
     for k, v in defines.items():
         cmd += f" -D{k}={v}"
     if link:
@@ -57,11 +67,11 @@ def compile_command(src, out, defines, link=""):
     return cmd
 
 
-def compile_library(src, out, defines, link=""):
+def compile_library(src, out, defines, link="", extra=""):
     """Returns (ok, stderr_text)."""
     os.makedirs(os.path.dirname(out), exist_ok=True)
     tmp = out + ".tmp"
-    proc = subprocess.run(compile_command(src, tmp, defines, link), shell=True, capture_output=True, text=True)
+    proc = subprocess.run(compile_command(src, tmp, defines, link, extra), shell=True, capture_output=True, text=True)
     if proc.returncode != 0:
         if os.path.exists(tmp):
             os.remove(tmp)
@@ -89,6 +99,20 @@ def parse_resource_usage(stderr_text):
     return out
 
 
+def total_scratch(usage):
+    """Scratch bytes per lane summed over the kernels of one library (parse_resource_usage's dict)."""
+    return sum(res.get("scratch", 0) for res in usage.values())
+
+
+def spills_less(usage, than):
+    """True when no kernel of `usage` has more scratch than the same kernel in `than` and the sum is smaller."""
+    if set(usage) != set(than):
+        return False
+    if any(usage[k].get("scratch", 0) > than[k].get("scratch", 0) for k in usage):
+        return False
+    return total_scratch(usage) < total_scratch(than)
+
+
 def resource_usage_path(directory):
     return os.path.join(directory, "resource_usage.json")
 
@@ -105,6 +129,14 @@ def compile_many(jobs, max_workers=None, progress=None):
 
     def run(job):
         ok, err = compile_library(*job)
+        if ok and total_scratch(parse_resource_usage(err)) > 0:
+            alt = job[1] + ".nosched"
+            ok_alt, err_alt = compile_library(job[0], alt, job[2], *job[3:4], extra=NO_SCHEDULER_OPTION)
+            if ok_alt and spills_less(parse_resource_usage(err_alt), parse_resource_usage(err)):
+                os.replace(alt, job[1])
+                err = err_alt
+            elif os.path.exists(alt):
+                os.remove(alt)
         return job, ok, err
 
     with ThreadPoolExecutor(max_workers=max_workers) as ex:

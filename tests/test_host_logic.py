@@ -3,6 +3,7 @@ stdout formats, dispatcher tables, and that every built library exports the whol
 import ctypes
 import glob
 import math
+import json
 import os
 import re
 import subprocess
@@ -310,6 +311,39 @@ def test_build_records_kernel_resources_and_conv_skips_spilling_gathers(monkeypa
     assert c16.conv_kernel_scratch(big, 64) == 52 and c16.conv_kernel_scratch(big, 24) == 0   # mode 2 spills, mode 1 has no record
     assert c16.cost_model(d, 100352, 256, 64, 64) == small      # the cheaper prediction is skipped: its gather spills
     assert c16.cost_model(d, 100352, 256, 72, 24) == big
+
+
+def test_spilling_library_is_rebuilt_without_the_scheduler(tmp_path, monkeypatch):
+    """compile_many builds a library whose kernels spill once more without the compiler's scheduler and keeps that
+    build when no kernel spills more in it and the sum is smaller; a library without spills is compiled once."""
+    remark = "x.hip:1:1: remark: Function Name: k%d [-Rpass-analysis=kernel-resource-usage]\n" \
+             "x.hip:1:1: remark:     ScratchSize [bytes/lane]: %d [-Rpass-analysis=kernel-resource-usage]\n"
+    calls = []
+    scratch = {("a.so", ""): (36, 48), ("a.so", helix_runtime.NO_SCHEDULER_OPTION): (0, 28),      # improves: kept
+               ("b.so", ""): (20, 8), ("b.so", helix_runtime.NO_SCHEDULER_OPTION): (0, 16),        # one kernel worse: dropped
+               ("c.so", ""): (0, 0)}                                                                # no spill: one build
+
+    def fake_compile(src, out, defines, link="", extra=""):
+        name = os.path.basename(out).replace(".nosched", "")
+        calls.append((name, extra))
+        with open(out, "w") as f:
+            f.write(extra or "default")
+        s0, s1 = scratch[(name, extra)]
+        return True, remark % (0, s0) + remark % (1, s1)
+
+    monkeypatch.setattr(helix_runtime, "compile_library", fake_compile)
+    jobs = [("x.hip", str(tmp_path / n), {}) for n in ("a.so", "b.so", "c.so")]
+    assert helix_runtime.compile_many(jobs, max_workers=2) == []
+    assert sorted(calls) == sorted([("a.so", ""), ("a.so", helix_runtime.NO_SCHEDULER_OPTION), ("b.so", ""),
+                                    ("b.so", helix_runtime.NO_SCHEDULER_OPTION), ("c.so", "")])
+    assert open(tmp_path / "a.so").read() == helix_runtime.NO_SCHEDULER_OPTION
+    assert open(tmp_path / "b.so").read() == "default" and open(tmp_path / "c.so").read() == "default"
+    assert not list(tmp_path.glob("*.nosched"))
+    usage = json.load(open(helix_runtime.resource_usage_path(str(tmp_path))))
+    assert usage["a.so"] == {"k0": {"scratch": 0}, "k1": {"scratch": 28}} and usage["b.so"]["k1"] == {"scratch": 8}
+    assert helix_runtime.spills_less({"k": {"scratch": 0}}, {"k": {"scratch": 4}})
+    assert not helix_runtime.spills_less({"k": {"scratch": 4}}, {"k": {"scratch": 4}})
+    assert not helix_runtime.spills_less({"k": {"scratch": 0}}, {"j": {"scratch": 4}})
 
 
 def test_fastdiv_header_matches_integer_division(tmp_path):
