@@ -1,4 +1,4 @@
-"""python3 benchmark_baseline_configs.py -c {square,gemv,conv,bert,all} -b <backend> [--oracle] [--no-tiles] [--vendor] [--json]
+"""python3 benchmark_baseline_configs.py -c {square,gemv,conv,bert,all} -b <backend> [--oracle] [--no-tiles] [--no-verified] [--vendor] [--json]
 
 The measured configurations of this backend, each against the roofline that bounds it:
   square  M = N = K in {1024, 2048, 4096, 8192}                              (MFMA peak)
@@ -89,7 +89,7 @@ def steady_vendor(be, M, N, K):
     return mn * 1e3, 2.0 * M * N * K / mn / 1e12
 
 
-def square_rows(be, prof_dict, oracle=False, vendor=False):
+def square_rows(be, prof_dict, oracle=False, vendor=False, verified=True):
     """Per size: the cost model's pick (Default) and the fastest of its first few candidates (Verified); oracle=True
     adds the exhaustive per-shape search, vendor=True rocBLAS on the same operand layouts."""
     rows = []
@@ -98,8 +98,9 @@ def square_rows(be, prof_dict, oracle=False, vendor=False):
         ms, tflops = steady_gemm(be, key, s, s, s)
         row = {"M": s, "N": s, "K": s, "config": list(key), "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
-        vms, vtf, vkey = steady_verified(be, prof_dict, key, ms, s, s, s)
-        row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
+        if verified:
+            vms, vtf, vkey = steady_verified(be, prof_dict, key, ms, s, s, s)
+            row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
         if oracle:
             oms, otf, okey = steady_oracle(be, prof_dict, key, ms, s, s, s)
             row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2),
@@ -151,7 +152,7 @@ def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
     return rows
 
 
-def conv_rows(be, prof_dict, vendor=False, oracle=False):
+def conv_rows(be, prof_dict, vendor=False, oracle=False, verified=True):
     """vendor=True adds MIOpen's time on the same layer (the comparator library); oracle=True the exhaustive
     per-layer search over every configuration with a conv entry (FP16 backend)."""
     miopen = load(be.build.kernel_library("miopen_f32" if be.fp32 else "miopen_f16")) if vendor else None
@@ -167,10 +168,11 @@ def conv_rows(be, prof_dict, vendor=False, oracle=False):
                      "TFLOP/s": round(tflops, 2), "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4),
                      "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / (ms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
-        vms, vtf, vkey = be.conv_verified(prof_dict, *shp)
-        if vms >= ms:   # the Default configuration is the first candidate
-            vms, vkey = ms, key
-        rows[-1].update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2)})
+        if verified:
+            vms, vtf, vkey = be.conv_verified(prof_dict, *shp)
+            if vms >= ms:   # the Default configuration is the first candidate
+                vms, vkey = ms, key
+            rows[-1].update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2)})
         if conv_oracle is not None:
             oms, otf, okey = conv_oracle(prof_dict, *shp)
             if oms >= ms:   # the Default configuration is one of the candidates
@@ -183,7 +185,7 @@ def conv_rows(be, prof_dict, vendor=False, oracle=False):
     return rows
 
 
-def bert_rows(be, prof_dict, oracle=False, vendor=False):
+def bert_rows(be, prof_dict, oracle=False, vendor=False, verified=True):
     """Per distinct GEMM of the encoder, then the whole list (12 layers + the irregular shape) as one row: summed
     latency, as the reference sums per-GEMM costs (benchmark_Ampere_FP16_model_level_LLM.py:16-27).  oracle=True adds
     the exhaustive per-shape search ("per-shape autotune"), vendor=True rocBLAS."""
@@ -198,9 +200,10 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
                    "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                    "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
             times = {"default": ms}
-            vms, vtf, vkey = steady_verified(be, prof_dict, dkey, ms, M, N, K)
-            row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
-            times["verified"] = vms
+            if verified:
+                vms, vtf, vkey = steady_verified(be, prof_dict, dkey, ms, M, N, K)
+                row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
+                times["verified"] = vms
             if oracle:
                 oms, otf, okey = steady_oracle(be, prof_dict, dkey, ms, M, N, K)
                 row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2)})
@@ -216,8 +219,9 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
         total_flops += 2.0 * M * N * K
     tf = total_flops / (totals["default"] * 1e-3) / 1e12
     total = {"total_ms": round(totals["default"], 4), "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf * 1e12 / be.peak, 4)}
-    vtf = total_flops / (totals["verified"] * 1e-3) / 1e12
-    total.update({"verified_total_ms": round(totals["verified"], 4), "verified_TFLOP/s": round(vtf, 2)})
+    if verified:
+        vtf = total_flops / (totals["verified"] * 1e-3) / 1e12
+        total.update({"verified_total_ms": round(totals["verified"], 4), "verified_TFLOP/s": round(vtf, 2)})
     if oracle:
         otf = total_flops / (totals["oracle"] * 1e-3) / 1e12
         total.update({"oracle_total_ms": round(totals["oracle"], 4), "oracle_TFLOP/s": round(otf, 2),
@@ -232,19 +236,19 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False):
 SECTIONS = {"square": square_rows, "gemv": gemv_rows, "conv": conv_rows, "bert": bert_rows}
 
 
-def run(backend, configs, oracle=False, tiles=True, vendor=False):
+def run(backend, configs, oracle=False, tiles=True, vendor=False, verified=True):
     be = Backend(backend)
     prof_dict = be.prof_dict()
     out = {}
     for name in configs:
         if name == "square":
-            out[name] = square_rows(be, prof_dict, oracle, vendor)
+            out[name] = square_rows(be, prof_dict, oracle, vendor, verified)
         elif name == "bert":
-            out[name] = bert_rows(be, prof_dict, oracle, vendor)
+            out[name] = bert_rows(be, prof_dict, oracle, vendor, verified)
         elif name == "gemv":
             out[name] = gemv_rows(be, prof_dict, tiles=tiles)
         elif name == "conv":
-            out[name] = conv_rows(be, prof_dict, vendor=vendor, oracle=oracle)
+            out[name] = conv_rows(be, prof_dict, vendor=vendor, oracle=oracle, verified=verified)
         else:
             out[name] = SECTIONS[name](be, prof_dict)
     return out
@@ -256,12 +260,13 @@ if __name__ == "__main__":
     parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default="MI355X_FP16")
     parser.add_argument("--oracle", action="store_true", help="square, bert, conv: also run the exhaustive per-shape search")
     parser.add_argument("--no-tiles", action="store_true", help="gemv: time the GEMV library only")
+    parser.add_argument("--no-verified", action="store_true", help="square, bert, conv: leave the Verified column out (Default launches only)")
     parser.add_argument("--vendor", action="store_true", help="conv: add MIOpen's time per layer; square, bert: add rocBLAS's")
     parser.add_argument("--json", action="store_true", help="one JSON object instead of the table")
     args = parser.parse_args()
 
     result = run(args.backend, list(SECTIONS) if args.config == "all" else [args.config], args.oracle,
-                 tiles=not args.no_tiles, vendor=args.vendor)
+                 tiles=not args.no_tiles, vendor=args.vendor, verified=not args.no_verified)
     if args.json:
         print(json.dumps(result))
     else:
