@@ -9,6 +9,7 @@ A step is one GEMM launch through the C ABI (helix_gemm) on operands already res
 one JSON line.
 """
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -71,7 +72,8 @@ def other_configs():
     for name in ("MI355X_FP16", "MI355X_FP32"):
         be = bc.Backend(name)
         t0 = time.perf_counter()
-        getattr(be.profile, f"profile_Helix_{name}_gemm_kernel")()
+        with contextlib.redirect_stdout(sys.stderr):     # the profile scripts' progress lines; stdout carries the one JSON line
+            getattr(be.profile, f"profile_Helix_{name}_gemm_kernel")()
         profile_s[name] = round(time.perf_counter() - t0, 2)
         dicts[name] = (be, read_prof_dict(name))
     out["profile_wall_s"] = profile_s
