@@ -67,7 +67,7 @@
 #define GEMV_KU2 8
 #endif
 #ifndef GEMV_R4
-#define GEMV_R4 2
+#define GEMV_R4 1
 #define GEMV_KU4 4
 #endif
 #ifndef GEMV_R8
@@ -88,7 +88,7 @@
 #define TARGET_WAVES 2048   // waves a launch aims for: 256 compute units x 8
 #endif
 #ifndef GEMV_MANY_WAVES_MT
-#define GEMV_MANY_WAVES_MT 2   // activation-row tiles up to this one run 16 waves per compute unit instead of 8
+#define GEMV_MANY_WAVES_MT 4   // activation-row tiles up to this one run 16 waves per compute unit instead of 8
 #endif
 #ifndef MFMA_MIN_M
 #define MFMA_MIN_M 9        // activation rows from which the MFMA variant takes over (measured crossover)
@@ -722,9 +722,9 @@ inline int launch_waves(Params p, int lds, hipStream_t s) {
 
 template <int MT, int ROWS, int KU>
 inline int launch_cfg(Params p, hipStream_t s) {
-    // One or two activation rows leave the vector units idle most of the time: twice the waves per CU, in workgroups
-    // of twice the size so that the activations are staged as often as before (measured 3 - 7 % on the decode shapes;
-    // slower from four rows on).
+    // Up to four activation rows leave the vector units idle most of the time: twice the waves per CU, in workgroups
+    // of twice the size so that the activations are staged as often as before (measured 3 - 8 % on the decode shapes;
+    // slower with the eight-row tile).
     const int lds = MT * p.kchunk * 2;
     const bool many = (MT <= GEMV_MANY_WAVES_MT) && lds <= X_LDS_BYTES;
     const long long target = many ? 2 * TARGET_WAVES : TARGET_WAVES;

@@ -32,8 +32,12 @@
 #define GEMV_KU2 8
 #endif
 #ifndef GEMV_R4
-#define GEMV_R4 2
+#define GEMV_R4 1
 #define GEMV_KU4 4
+#endif
+#ifndef GEMV_R4_WIDE
+#define GEMV_R4_WIDE 2
+#define GEMV_KU4_WIDE 4
 #endif
 #ifndef GEMV_R8
 #define GEMV_R8 4
@@ -50,7 +54,7 @@
 #define X_LDS_BYTES_WIDE 131072   // ... of one workgroup of twice as many waves, alone on its CU: same waves per CU
 #endif
 #ifndef GEMV_MANY_WAVES_MT
-#define GEMV_MANY_WAVES_MT 2   // activation-row tiles up to this one run 16 waves per compute unit instead of 8
+#define GEMV_MANY_WAVES_MT 4   // activation-row tiles up to this one run 16 waves per compute unit instead of 8
 #endif
 #ifndef TARGET_WAVES
 #define TARGET_WAVES 2048   // waves a launch aims for: 256 compute units x 8
@@ -358,9 +362,9 @@ inline int launch_waves(Params p, int lds, hipStream_t s) {
 
 template <int MT, int ROWS, int KU>
 inline int launch_cfg(Params p, hipStream_t s) {
-    // One or two activation rows leave the vector units idle most of the time: twice the waves per CU, in workgroups
-    // of twice the size so that the activations are staged as often as before (measured 2 - 7 % on the decode shapes;
-    // slower from four rows on).
+    // Up to four activation rows leave the vector units idle most of the time: twice the waves per CU, in workgroups
+    // of twice the size so that the activations are staged as often as before (measured 2 - 13 % on the decode shapes;
+    // slower with the eight-row tile).
     const int lds = MT * p.kchunk * 4;
     const bool many = (MT <= GEMV_MANY_WAVES_MT) && lds <= X_LDS_BYTES;
     const long long target = many ? 2 * TARGET_WAVES : TARGET_WAVES;
@@ -390,7 +394,12 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     switch (mtile_of(M)) {
         case 1: rc = launch_cfg<1, GEMV_R1, GEMV_KU1>(p, s); break;
         case 2: rc = launch_cfg<2, GEMV_R2, GEMV_KU2>(p, s); break;
-        case 4: rc = launch_cfg<4, GEMV_R4, GEMV_KU4>(p, s); break;
+        case 4:
+            // four rows: one weight row per pass while the staged activations leave room for 16 waves per CU
+            // (3 - 13 % faster there), two rows per pass when they fill the LDS and 8 waves share them
+            if (4 * p.kchunk * 4 <= X_LDS_BYTES) rc = launch_cfg<4, GEMV_R4, GEMV_KU4>(p, s);
+            else rc = launch_cfg<4, GEMV_R4_WIDE, GEMV_KU4_WIDE>(p, s);
+            break;
         case 8: rc = launch_cfg<8, GEMV_R8, GEMV_KU8>(p, s); break;
         default: rc = launch_cfg<16, GEMV_R16, GEMV_KU16>(p, s); break;
     }
