@@ -39,7 +39,8 @@
 //     spans, the pattern that streams fastest -- and the MFMA operands (lane l: row l % 16, columns 8*(l/16) .. +7 of
 //     a 32-wide block) are read back from LDS.  Loading the operand layout straight into registers (16 rows x 64
 //     bytes per instruction) measured 4.3 TB/s on 8192 x 28672 weights at 16 rows, this variant 5.8;
-//   * eight MFMAs per step accumulate the 16 x 16 block y[m][n]; copies run three steps ahead; buffer bounds
+//   * eight MFMAs per step accumulate the 16 x 16 block y[m][n]; copies run two steps ahead (a ring of three slots measured
+//     as fast as or up to 4 % faster than four); buffer bounds
 //     checking zero-fills weight rows beyond N;
 //   * two work splits: a wave owns its own row groups and all columns of the K range, or the four waves of a
 //     workgroup share their groups, take a quarter of every staged chunk each and add their sums through LDS at the
@@ -344,7 +345,7 @@ constexpr int MGROUPS = 8;                      // most 16-row groups one wave o
 // the workgroup's activation staging and from one 16-row group to the next.
 constexpr int SSTEP = 256;                       // columns per step
 #ifndef STREAM_RING
-#define STREAM_RING 4
+#define STREAM_RING 3
 #endif
 #ifndef STREAM_XC
 #define STREAM_XC 512
