@@ -15,10 +15,11 @@ from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K, PROFILE_K_SHORT
 root_path = os.getcwd()
 
 HBM_SUSTAINED_FRACTION = 0.8  # share of the datasheet HBM rate a streaming kernel sustains
-# ... and what the tile kernels sustain when a problem is a pass over a cold operand (measured 5.2 - 5.5 TB/s on
-# 8192 x 28672 weights): their profile point is a hot 16 x 16-tile problem, so this floor is what ranks them against
-# the weight-streaming kernels, whose profile point is cold
-TILE_HBM_SUSTAINED_FRACTION = 0.68
+# ... and what the tile kernels sustain when a problem is a pass over a cold operand (on 8192 x 28672 weights the
+# fastest 32-row tile measures 5.2 - 5.5 TB/s, the one the model ranks first 4.4 - 4.9): their profile point is a hot
+# 16 x 16-tile problem, so this floor is what ranks them against the weight-streaming kernels, whose profile point
+# is cold
+TILE_HBM_SUSTAINED_FRACTION = 0.60
 GEMV_LAUNCH_FLOOR_S = 3.4e-6       # a kernel launch on an idle queue; keeps tiny problems from looking free
 GEMV_MFMA_FLOOR_S = 4.4e-6         # 9 or more activation rows: the LDS-streamed MFMA variant (staging + cross-wave sum)
 GEMV_MFMA_MIN_M = 9                # MFMA_MIN_M of src_template/MI355X_FP16/gemv.hip

@@ -216,7 +216,10 @@ def test_fp16_cost_model_two_point_profile():
                                       roofline.gemm_bytes(100352, 256, 64, 2) / (g16.TILE_HBM_SUSTAINED_FRACTION * roofline.HBM_BYTES_PER_S)))
     assert g16.cost_model(d, 100352, 256, 64) == big
     # without the short point a round is taken to cost K / K_profile of the profiled one: 49 almost free rounds
-    assert g16.config_cost(small, d[small], 100352, 256, 64) == pytest.approx(49 * 17e-6 * 64 / K)
+    hbm_floor = roofline.gemm_bytes(100352, 256, 64, 2) / (g16.TILE_HBM_SUSTAINED_FRACTION * roofline.HBM_BYTES_PER_S)
+    assert g16.config_cost(small, d[small], 100352, 256, 64) == pytest.approx(max(49 * 17e-6 * 64 / K, hbm_floor))
+    assert 49 * 17e-6 * 64 / K < hbm_floor < 49 * 17e-6 * 128 / K          # the floor binds for this shape, not for twice its K
+    assert g16.config_cost(small, d[small], 100352, 256, 128) == pytest.approx(49 * 17e-6 * 128 / K)
     # conv: every column of tiles gathers its rows again
     assert c16.conv_config_cost(big, 60e-6, 4096, 512, K, 8e-6) == \
         pytest.approx(g16.config_cost(big, 60e-6, 4096, 512, K, 8e-6) * (1 + 2 * c16.GATHER_COST_PER_TILE_COLUMN))
