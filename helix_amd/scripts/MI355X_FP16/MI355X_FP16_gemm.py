@@ -161,12 +161,14 @@ def get_MI355X_FP16_gemm_rocblas_result(M, N, K):
 def get_MI355X_FP16_gemm_Verified_result(prof_dict, M, N, K, top=VERIFY_TOP):
     """The fastest of the cost model's first `top` configurations: each timed briefly, the winner timed again with
     the runner's launch counts.  Returns (cost_ms, tflops, key)."""
-    timed = []
+    timed, last_error = [], None
     for k in ranked_configs(prof_dict, M, N, K, top):
         try:
             timed.append((run_config(k, M, N, K, warmup=2, iters=5), k))
-        except Exception:
-            continue
+        except Exception as e:     # a candidate that cannot run this shape is skipped, as the profile skips it
+            last_error = e
+    if not timed:
+        raise RuntimeError(f"none of the {top} ranked configurations could run {M}x{N}x{K}") from last_error
     best = min(timed)[1]
     cost = run_config(best, M, N, K)
     return cost * 1e3, 2 * M * N * K / 1e12 / cost, best

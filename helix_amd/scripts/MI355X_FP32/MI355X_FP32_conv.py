@@ -57,14 +57,17 @@ def get_MI355X_FP32_conv_Verified_result(prof_dict, batch, input_channel, H, W, 
     again with the runner's launch counts.  Returns (cost_ms, tflops, key)."""
     M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
     flops = 2.0 * M * output_channel * input_channel * kH * kW
-    timed = []
+    timed, last_error = [], None
     for k in ranked_configs(prof_dict, M, output_channel, gather_channels(input_channel) * kH * kW, top):
         try:
             _, avg, _ = load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride,
                                                             pad, warmup=2, iters=5)
-        except Exception:
+        except Exception as e:     # a candidate that cannot run this layer is skipped, as the profile skips it
+            last_error = e
             continue
         timed.append((avg, k))
+    if not timed:
+        raise RuntimeError(f"none of the {top} ranked configurations could run this layer") from last_error
     best = min(timed)[1]
     _, cost, _ = load(library_for_key(best)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
                                                         warmup=10, iters=10)

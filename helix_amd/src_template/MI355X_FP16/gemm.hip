@@ -641,4 +641,7 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
 
 }  // namespace tpl
 
+#if SPLIT_K == 1
+#define HELIX_TPL_SCRATCH_BYTES 256   // no K partition: this library never asks for a workspace
+#endif
 #include "helix_host.h"

@@ -8,8 +8,9 @@
 // waves divide the work:
 //   * global memory -> LDS without passing through registers (buffer_load ... lds: one wave-wide instruction
 //     writes 1 KiB of consecutive LDS), into a ring of K_STAGES stages of BLOCK_K (32, 64 or 128) columns;
-//   * a workgroup is eight waves, two on each SIMD.  On arrival each wave takes a ticket per SIMD: the first
-//     wave of a SIMD joins group 0, the second group 1.  A wave alternates between two phases per K tile,
+//   * a workgroup is eight waves, normally two on each SIMD.  On arrival each wave takes a ticket per SIMD: the first
+//     wave of a SIMD joins group 0, the second group 1 (if the waves are not spread two per SIMD, groups and copy
+//     quarters are dealt by wave index instead).  A wave alternates between two phases per K tile,
 //       M(t): read its fragments of tile t (the whole tile: KSTEPS x (TM + TN) ds_read_b128) into registers,
 //       C(t): KSTEPS x TM x TN MFMAs on those registers, nothing else,
 //     with a workgroup barrier behind every phase, and group 1 runs one phase behind group 0.  So on every SIMD
@@ -124,10 +125,19 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_dtl_kernel(const Para
     if (tid < 4) role[tid] = 0;
     __syncthreads();
     // HW_REG_HW_ID (register 4), SIMD_ID = bits 5:4
-    const int simd = __builtin_amdgcn_s_getreg((2 - 1) << 11 | 4 << 6 | 4) & 3;
+    const int hw_simd = __builtin_amdgcn_s_getreg((2 - 1) << 11 | 4 << 6 | 4) & 3;
     int ticket = 0;
-    if (lane == 0) ticket = atomicAdd(&role[simd], 1);
-    const int grp = __builtin_amdgcn_readfirstlane(ticket) & 1;
+    if (lane == 0) ticket = atomicAdd(&role[hw_simd], 1);
+    __syncthreads();
+    // The dispatcher usually places two of the eight waves on each SIMD, and then the tickets give every SIMD one
+    // wave of each group.  Nothing guarantees that placement (small tiles share a compute unit with other
+    // workgroups): when the counts are not 2 / 2 / 2 / 2 the groups and the copy quarters are dealt by wave index
+    // instead, which is correct under any placement (the two waves of a SIMD may then be in the same phase).
+    const bool two_per_simd = role[0] == 2 && role[1] == 2 && role[2] == 2 && role[3] == 2;
+    // wave-uniform values, kept in scalar registers (lane 0 holds the ticket)
+    const int grp = __builtin_amdgcn_readfirstlane(two_per_simd ? (ticket & 1) : (wave & 1));
+    // the quarter of every stage a group-0 wave copies
+    const int simd = __builtin_amdgcn_readfirstlane(two_per_simd ? hw_simd : (wave >> 1));
 
     // ---- copy geometry of a group-0 wave: quarter `simd` of the A rows and of the B rows of every stage ----------
     // Copy instruction j fills LRPI consecutive LDS rows (1 KiB) from LDS row q / MPL + j * LRPI on; lane l lands at
@@ -344,4 +354,7 @@ inline int conv2d(const void*, const void*, void*, int, int, int, int, int, int,
 
 }  // namespace tpl
 
+#if SPLIT_K == 1
+#define HELIX_TPL_SCRATCH_BYTES 256   // no K partition: this library never asks for a workspace
+#endif
 #include "helix_host.h"

@@ -520,8 +520,10 @@ __global__ __launch_bounds__(64 * SWPB) void helix_gemv_f16_mfma_stream_kernel(c
 
     for (int kc = k_begin; kc < k_end; kc += SXC) {
         __syncthreads();                                              // the previous chunk has been read
-        // loads complete in order: the chunk's activations are older than the steps_after_x newest weight steps
-        wait_steps_in_flight<0>(steps_after_x);
+        // loads complete in order: the chunk's activations are older than the weight steps issued behind them, of
+        // which at most issued - used are still in flight (a larger count would read as "wait for everything" and
+        // drain the ring)
+        wait_steps_in_flight<0>(steps_after_x < issued - used ? steps_after_x : issued - used);
 #pragma unroll
         for (int i = 0; i < XPT; i++) {
             const int c = tid + i * (64 * SWPB);

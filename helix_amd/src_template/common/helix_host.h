@@ -162,7 +162,15 @@ int helix_conv2d(const void* x, const void* w, void* y, int batch, int H, int W,
 // a caller-provided workspace.  Every GPU the library runs on holds its own copy of the array, at its own
 // address, until the process ends.  In host code the name is only a handle for HIP_SYMBOL(); the memory is
 // reached through the per-device pointer below.
-static __device__ __align__(256) unsigned char scratch[HELIX_STATIC_SCRATCH_BYTES];
+//
+// HELIX_TPL_SCRATCH_BYTES (a template may define it before including this file) is the size this library gives the
+// array: HELIX_STATIC_SCRATCH_BYTES unless the template never asks for a workspace (tpl::workspace_bytes is 0 for
+// every shape), in which case a token array keeps the symbol and the entry point's code path the same.
+#ifndef HELIX_TPL_SCRATCH_BYTES
+#define HELIX_TPL_SCRATCH_BYTES HELIX_STATIC_SCRATCH_BYTES
+#endif
+static_assert(HELIX_TPL_SCRATCH_BYTES <= HELIX_STATIC_SCRATCH_BYTES, "the documented maximum bounds every library");
+static __device__ __align__(256) unsigned char scratch[HELIX_TPL_SCRATCH_BYTES];
 
 namespace helix_host {
 namespace {
@@ -194,13 +202,13 @@ int helix_gemm_static_scratch(const void* A, const void* B, void* C, int M, int 
                               void* stream) {
     if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return HELIX_ERR_INVALID_VALUE;
     const size_t need = tpl::workspace_bytes(M, N, K);
-    if (need > (size_t)HELIX_STATIC_SCRATCH_BYTES) return HELIX_ERR_WORKSPACE;
+    if (need > (size_t)HELIX_TPL_SCRATCH_BYTES) return HELIX_ERR_WORKSPACE;
     void* ws = nullptr;
     int rc = helix_host::static_scratch(&ws);
     if (rc) return rc;
     // Nothing to clear: a K-partitioned launch writes every partial sum of its M x N x partitions block before
     // its reduction pass reads that block, and reads nothing else of the array.
-    return tpl::gemm(A, B, C, M, N, K, lda, ldb, ldc, ws, (size_t)HELIX_STATIC_SCRATCH_BYTES, (hipStream_t)stream);
+    return tpl::gemm(A, B, C, M, N, K, lda, ldb, ldc, ws, (size_t)HELIX_TPL_SCRATCH_BYTES, (hipStream_t)stream);
 }
 #else
 int helix_gemm_static_scratch(const void*, const void*, void*, int, int, int, int, int, int, void*) {

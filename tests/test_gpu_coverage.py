@@ -103,6 +103,33 @@ def test_every_fp16_library_integer_exact(keys):
             assert np.array_equal(got.astype(np.float32), exact), (key, x.shape, w.shape)
 
 
+def test_many_tile_grids_integer_exact():
+    """An integer-valued 4096 x 4096 x 256 GEMM: a few thousand tiles, so that workgroups of the small tiles share
+    compute units and their waves arrive in whatever placement the dispatcher produces.  Every direct-to-LDS
+    configuration (its wave groups and copy quarters are dealt by placement, with a placement-independent deal as
+    the fallback) and every eighth register-staged one; the whole result is compared on the device with the exact
+    product, which a corner block ties to int64 arithmetic on the host."""
+    M = N = 4096
+    K = 256
+    rng = np.random.default_rng(7)
+    A = rng.integers(-2, 3, (M, K)).astype(np.float16)
+    Bt = rng.integers(-1, 2, (N, K)).astype(np.float16)
+    dA, dBt = dev(A), dev(Bt)
+    want = (dA.float() @ dBt.float().T)          # integers below 2^24: exact in FP32 in any summation order
+    assert float(want.abs().max()) <= 2 * K
+    corner = A[:300].astype(np.int64) @ Bt[:300].astype(np.int64).T
+    assert np.array_equal(want[:300, :300].cpu().numpy().astype(np.int64), corner)
+    want16 = want.half()
+    dtl = [k for k in FP16_TILE_KEYS if b16.is_dtl_key(k)]
+    staged = [k for k in FP16_TILE_KEYS if not b16.is_dtl_key(k)][::8]
+    assert len(dtl) >= 2 and len(staged) > 30
+    for key in dtl + staged:
+        lib = load(b16.library_for_key(key))
+        for _ in range(2):                       # twice: placements differ from launch to launch
+            got = run_gemm_f16_dev(lib, dA, dBt, M, N, K, K)
+            assert torch.equal(got, want16), (key, int((got != want16).sum()))
+
+
 @pytest.mark.parametrize("keys", _chunks(FP32_TILE_KEYS), ids=lambda ks: f"{ks[0]}..")
 def test_every_fp32_library_integer_exact(keys):
     """Per configuration: the same GEMMs with and without the K-partition workspace, and convolutions with

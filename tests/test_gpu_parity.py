@@ -150,14 +150,32 @@ def test_gemm_f16_golden_vectors():
         assert normwise(got, O.hgemm_f32acc(d["A"], d["B"])) < TOL16, f
 
 
-def test_gemm_f16_full_size_properties():
+# the 256 x 256-tile configurations the search's winner at 8192^3 has come from (register-staged and direct-to-LDS)
+FULL_SIZE_KEYS = [(2, 256, 256, 64, 128, 0, 64), (2, 256, 256, 128, 64, 0, 64), (2, 256, 256, 128, 128, 0, 64),
+                  (2, 256, 256, 64, 128, 0, 64, 1), (2, 256, 256, 128, 64, 0, 64, 1)]
+
+
+@pytest.fixture(scope="module")
+def full_size_operands():
+    M = N = K = 8192
+    A, B = seeded_inputs.gemm_operands(M, N, K, np.float16)
+    Bt = np.ascontiguousarray(B.T)
+    return A, Bt, dev(A), dev(Bt)
+
+
+def test_full_size_keys_cover_the_benchmark_candidates():
+    """The configurations bench.py knows counted traffic for (its winners so far) are the ones tested at full size."""
+    import bench
+    assert set(FULL_SIZE_KEYS) == set(bench.MEASURED_TRAFFIC)
+
+
+@pytest.mark.parametrize("key", FULL_SIZE_KEYS, ids=lambda k: "_".join(map(str, k)))
+def test_gemm_f16_full_size_properties(key, full_size_operands):
     """8192^3 (the benchmark size): too big for the CPU oracle in seconds, so check size-independent facts:
     a random sample of outputs against float64 dot products, and linearity in A."""
     M = N = K = 8192
-    lib = load(b16.kernel_library("gemm", 2, 256, 256, 128, 128, 64))
-    A, B = seeded_inputs.gemm_operands(M, N, K, np.float16)
-    Bt = np.ascontiguousarray(B.T)
-    dA, dB = dev(A), dev(Bt)
+    lib = load(b16.library_for_key(key))
+    A, Bt, dA, dB = full_size_operands
     dC = torch.empty((M, N), dtype=torch.float16, device="cuda:0")
     lib.gemm(dA.data_ptr(), dB.data_ptr(), dC.data_ptr(), M, N, K, K, K, N)
     torch.cuda.synchronize()

@@ -186,6 +186,34 @@ def test_static_cost_models():
     assert cmp16.cost_model_static2(d, 64, 64, 64) == (2, 256, 128, 64, 64, 0, 64)         # best time per tile area
 
 
+def test_verified_selection_reports_why_no_candidate_ran(monkeypatch):
+    """When every ranked candidate fails, Verified mode raises an error that carries the last failure instead of
+    min() over an empty list."""
+    d16 = {(2, 128, 128, 64, 64, 0, 64): 1.0, (2, 64, 64, 64, 64, 0, 64): 0.4}
+    d32 = {b32.config_key(64, 64, 16, 32, 32): 1.0}
+
+    def failing(*a, **kw):
+        raise hip_ctypes.HelixError("helix_bench", 100)
+
+    monkeypatch.setattr(g16, "run_config", failing)
+    monkeypatch.setattr(g32, "run_config", failing)
+    for fn, d in ((g16.get_MI355X_FP16_gemm_Verified_result, d16), (g32.get_MI355X_FP32_gemm_Verified_result, d32)):
+        with pytest.raises(RuntimeError, match="ranked configurations could run 64x64x64") as info:
+            fn(d, 64, 64, 64)
+        assert isinstance(info.value.__cause__, hip_ctypes.HelixError) and info.value.__cause__.code == 100
+
+    class Failing:
+        def bench_conv(self, *a, **kw):
+            raise hip_ctypes.HelixError("helix_bench_conv", 100)
+
+    monkeypatch.setattr(c16, "load", lambda path: Failing())
+    monkeypatch.setattr(c32, "load", lambda path: Failing())
+    for fn, d in ((c16.get_MI355X_FP16_conv_Verified_result, d16), (c32.get_MI355X_FP32_conv_Verified_result, d32)):
+        with pytest.raises(RuntimeError, match="ranked configurations could run this layer") as info:
+            fn(d, 1, 8, 8, 8, 8, 3, 3, 1, 1)
+        assert isinstance(info.value.__cause__, hip_ctypes.HelixError)
+
+
 def test_fp32_cost_model_hand_cases():
     K = p32.PROFILE_K
     d = {(128, 128, 16, 64, 64, 2, 1, 4): 1.0, (256, 128, 16, 128, 64, 2, 1, 4): 1.8}

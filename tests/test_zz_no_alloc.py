@@ -86,3 +86,24 @@ def test_static_scratch_limit_and_refusals():
     for path in (b16.kernel_library("rocblas_f16"), b32.kernel_library("rocblas_f32")):
         assert load(path).gemm_static_scratch(A.data_ptr(), A.data_ptr(), C.data_ptr(), 64, 64, 64, K, K, N,
                                               check=False) == HELIX_ERR_UNSUPPORTED
+
+
+def test_static_scratch_call_allocates_no_device_memory():
+    """The property the entry point exists for: after a warm-up call (the first launch of a library loads its code
+    object, scratch array included), further calls leave the device's free memory unchanged."""
+    lib = load(b16.kernel_library("gemm_splitK", 2, 64, 64, 32, 32, 64))
+    M, N, K = 320, 448, 4096
+    A = torch.ones((M, K), dtype=torch.float16, device="cuda:0")
+    B = torch.ones((N, K), dtype=torch.float16, device="cuda:0")
+    C = torch.empty((M, N), dtype=torch.float16, device="cuda:0")
+    assert 0 < lib.workspace_bytes(M, N, K) <= STATIC_SCRATCH_BYTES
+    stream = torch.cuda.current_stream().cuda_stream
+    lib.gemm_static_scratch(A.data_ptr(), B.data_ptr(), C.data_ptr(), M, N, K, K, K, N, stream)   # warm-up
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for (m, n) in [(M, N), (130, 72), (M, N), (64, 448)]:
+        lib.gemm_static_scratch(A.data_ptr(), B.data_ptr(), C.data_ptr(), m, n, K, K, K, N, stream)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    assert bool((C[:64, :448] == K).all())
