@@ -11,7 +11,7 @@ repack + GEMM), all on one stream and timed as one.
 import math
 import os
 
-from utils.helix_runtime import load, kernel_resources
+from utils.helix_runtime import load, kernel_resources, tuned_config
 from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, is_dtl_key
 from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, VERIFY_TOP
 
@@ -111,12 +111,9 @@ def ranked_configs(prof_dict, M, N, K, IC=None, top=VERIFY_TOP):
     return [k for _, k in cand[:top]]
 
 
-def get_MI355X_FP16_conv_Verified_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
-                                         top=VERIFY_TOP):
-    """The fastest of the cost model's first `top` configurations on this layer: each timed briefly, the winner timed
-    again with the runner's launch counts.  Returns (cost_ms, tflops, key)."""
+def verified_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, top=VERIFY_TOP):
+    """The fastest of the cost model's first `top` configurations on this layer, each timed with 2 + 5 launches."""
     M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
-    flops = 2.0 * M * output_channel * input_channel * kH * kW
     ICg = gather_channels(input_channel)
     timed, last_error = [], None
     for k in ranked_configs(prof_dict, M, output_channel, ICg * kH * kW, ICg, top):
@@ -129,10 +126,31 @@ def get_MI355X_FP16_conv_Verified_result(prof_dict, batch, input_channel, H, W, 
         timed.append((avg, k))
     if not timed:
         raise RuntimeError(f"none of the {top} ranked configurations could run this layer") from last_error
-    best = min(timed)[1]
+    return min(timed)[1]
+
+
+def get_MI355X_FP16_conv_Verified_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
+                                         top=VERIFY_TOP):
+    """The fastest of the cost model's first `top` configurations on this layer: each timed briefly, the winner timed
+    again with the runner's launch counts.  Returns (cost_ms, tflops, key)."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    flops = 2.0 * M * output_channel * input_channel * kH * kW
+    best = verified_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, top)
     _, cost, _ = load(library_for_key(best)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
                                                         warmup=10, iters=10)
     return cost * 1e3, flops / 1e12 / cost, best
+
+
+def select_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
+    """The configuration the runner launches for this layer: the cost model's ranking, settled on the device the first
+    time the layer is met and remembered beside the profile (utils.helix_runtime.tuned_config); the cost model's
+    first choice alone with HELIX_SELECTION=model."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    ICg = gather_channels(input_channel)
+    layer = (batch, input_channel, H, W, output_channel, kH, kW, stride, pad)
+    return tuned_config("MI355X_FP16", ("conv",) + layer, prof_dict,
+                        lambda: cost_model(prof_dict, M, output_channel, ICg * kH * kW, ICg),
+                        lambda: verified_config(prof_dict, *layer))
 
 
 def get_MI355X_FP16_conv_Helix_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
@@ -142,7 +160,7 @@ def get_MI355X_FP16_conv_Helix_result(prof_dict, batch, input_channel, H, W, out
     M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
     N = output_channel
     K = input_channel * kH * kW
-    best_config = cost_model(prof_dict, M, N, gather_channels(input_channel) * kH * kW, gather_channels(input_channel))
+    best_config = select_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad)
     lib = load(library_for_key(best_config))
     _, avg, _ = lib.bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad, warmup=10, iters=10)
     cost = avg * 1e3

@@ -31,7 +31,8 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
                             pbar.update(1)
                             if splitK == 1 and K_STAGES not in SPLITK_STAGES_LIST:
                                 continue
-                            if not is_valid_config(1, 1, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES):
+                            if not is_valid_config(1, 1, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES,
+                                                   splitK):
                                 continue
                             base_key = (K_STAGES, WAVE_ROWS, WAVE_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K)
                             cost = time_config(base_key)
@@ -41,7 +42,7 @@ def profile_Helix_MI355X_FP16_gemm_kernel():
                                     BLOCK_ROWS = BLOCK_ROWS_SCALE * WAVE_ROWS
                                     BLOCK_COLS = BLOCK_COLS_SCALE * WAVE_COLS
                                     if not is_valid_config(BLOCK_ROWS_SCALE, BLOCK_COLS_SCALE, BLOCK_ROWS, BLOCK_COLS,
-                                                           WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES):
+                                                           WAVE_ROWS, WAVE_COLS, BLOCK_K, K_STAGES, splitK):
                                         continue
                                     key = (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, splitK, BLOCK_K)
                                     prof_dict[key] = float(cost) * BLOCK_ROWS_SCALE * BLOCK_COLS_SCALE

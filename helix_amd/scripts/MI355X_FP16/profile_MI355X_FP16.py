@@ -14,7 +14,7 @@ from tqdm import tqdm
 
 from utils.helix_runtime import load, write_prof_dict, ProfDict, kernel_resources
 from utils.roofline import NUM_CU
-from MI355X_FP16.build_MI355X_FP16 import iter_configs, iter_dtl_configs, library_for_key, SPLITK_STAGES_LIST
+from MI355X_FP16.build_MI355X_FP16 import iter_configs, iter_splitk_configs, iter_dtl_configs, library_for_key
 
 root_path = os.getcwd()
 
@@ -71,8 +71,8 @@ def all_keys():
         if K_STAGES > 2 and gemm_kernel_scratch(key) > 0:
             continue
         keys.append(key)
-        if K_STAGES in SPLITK_STAGES_LIST:
-            keys.append((K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 1, BLOCK_K))
+    for (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in iter_splitk_configs():
+        keys.append((K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 1, BLOCK_K))
     for (K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, BLOCK_K) in iter_dtl_configs():
         keys.append((K_STAGES, BLOCK_ROWS, BLOCK_COLS, WAVE_ROWS, WAVE_COLS, 0, BLOCK_K, 1))   # direct-to-LDS family
     keys.extend(GEMV_KEYS)

@@ -4,7 +4,7 @@ the TVM alternative backend (:16-86, :108-136) has no counterpart."""
 import math
 import os
 
-from utils.helix_runtime import load
+from utils.helix_runtime import load, tuned_config
 from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
 from MI355X_FP32.build_MI355X_FP32 import library_for_key, kernel_library
 from MI355X_FP32.profile_MI355X_FP32 import PROFILE_K, PROFILE_K_SHORT, GEMV_PROFILE_K
@@ -155,10 +155,31 @@ def run_config(k, M, N, K, warmup=10, iters=10, outer=1):
     return avg
 
 
+def verified_config(prof_dict, M, N, K, top=VERIFY_TOP):
+    """The fastest of the cost model's first `top` configurations on this problem, each timed with 2 + 5 launches."""
+    timed, last_error = [], None
+    for k in ranked_configs(prof_dict, M, N, K, top):
+        try:
+            timed.append((run_config(k, M, N, K, warmup=2, iters=5), k))
+        except Exception as e:     # a candidate that cannot run this shape is skipped, as the profile skips it
+            last_error = e
+    if not timed:
+        raise RuntimeError(f"none of the {top} ranked configurations could run {M}x{N}x{K}") from last_error
+    return min(timed)[1]
+
+
+def select_config(prof_dict, M, N, K):
+    """The configuration the runner launches: the cost model's ranking, settled on the device the first time a
+    problem is met and remembered beside the profile (utils.helix_runtime.tuned_config); the cost model's first
+    choice alone with HELIX_SELECTION=model."""
+    return tuned_config("MI355X_FP32", ("gemm", M, N, K), prof_dict, lambda: cost_model(prof_dict, M, N, K),
+                        lambda: verified_config(prof_dict, M, N, K))
+
+
 def get_MI355X_FP32_gemm_Helix_result(prof_dict, M, N, K, backend="hip"):
     if backend != "hip":
         raise ValueError(f"backend {backend!r} is not available for MI355X_FP32 (only 'hip')")
-    best_config = cost_model(prof_dict, M, N, K)
+    best_config = select_config(prof_dict, M, N, K)
     cost = run_config(best_config, M, N, K) * 1e3
     tflops = 2 * M * N * K / 1e9 / cost
 
@@ -177,15 +198,7 @@ def get_MI355X_FP32_gemm_rocblas_result(M, N, K):
 def get_MI355X_FP32_gemm_Verified_result(prof_dict, M, N, K, top=VERIFY_TOP):
     """The fastest of the cost model's first `top` configurations: each timed briefly, the winner timed again with
     the runner's launch counts.  Returns (cost_ms, tflops, key)."""
-    timed, last_error = [], None
-    for k in ranked_configs(prof_dict, M, N, K, top):
-        try:
-            timed.append((run_config(k, M, N, K, warmup=2, iters=5), k))
-        except Exception as e:     # a candidate that cannot run this shape is skipped, as the profile skips it
-            last_error = e
-    if not timed:
-        raise RuntimeError(f"none of the {top} ranked configurations could run {M}x{N}x{K}") from last_error
-    best = min(timed)[1]
+    best = verified_config(prof_dict, M, N, K, top)
     cost = run_config(best, M, N, K)
     return cost * 1e3, 2 * M * N * K / 1e12 / cost, best
 

@@ -5,9 +5,11 @@ The measured configurations of this backend, each against the roofline that boun
   gemv    decode shapes, M in {1, 4, 16} activation rows, weights cold       (HBM peak)
   conv    batch-32 NHWC ResNet-50-shaped layers, implicit GEMM               (MFMA peak and HBM peak)
   bert    BERT-base encoder GEMMs at 4096 tokens x 12 layers + 4000x2300x770 (MFMA peak)
-Every row is run through the cost model's pick (what the reference's benchmark wrappers do,
-scripts/Ampere_FP16/benchmark_Ampere_FP16_gemm.py:9-30); --oracle adds the exhaustive per-shape search
-(benchmark_Ampere_FP16_performance_comparison.py:56-69).  Needs build_template.py to have run; profiles
+Every row is run through the runner's selection, as the reference's benchmark wrappers do
+(scripts/Ampere_FP16/benchmark_Ampere_FP16_gemm.py:9-30): the cost model's ranking settled on the device and
+remembered per problem (select_config), with the cost model's first choice alone beside it (model_config, model_us)
+where the two differ; --no-verified runs the cost model's first choice only.  --oracle adds the exhaustive per-shape
+search (benchmark_Ampere_FP16_performance_comparison.py:56-69).  Needs build_template.py to have run; profiles
 first when no cost-model dict is on disk.
 """
 import argparse
@@ -34,8 +36,6 @@ class Backend:
                                                          mod(f"build_{name}"), mod(f"profile_{name}"))
         self.gemm_result = getattr(self.gemm, f"get_{name}_gemm_Helix_result")
         self.gemm_oracle = getattr(self.gemm, f"get_{name}_gemm_Oracle_result")
-        self.gemm_verified = getattr(self.gemm, f"get_{name}_gemm_Verified_result")
-        self.conv_verified = getattr(self.conv, f"get_{name}_conv_Verified_result")
         self.conv_result = getattr(self.conv, f"get_{name}_conv_Helix_result")
         self.gemm_vendor = getattr(self.gemm, f"get_{name}_gemm_rocblas_result")
 
@@ -72,15 +72,10 @@ def steady_oracle(be, prof_dict, dkey, dms, M, N, K):
     return dms, 2.0 * M * N * K / (dms * 1e-3) / 1e12, dkey
 
 
-def steady_verified(be, prof_dict, dkey, dms, M, N, K):
-    """(ms, TFLOP/s, key) of Verified mode (the fastest of the cost model's first few candidates, the Default
-    configuration among them), timed like the Default column."""
-    _, _, vkey = be.gemm_verified(prof_dict, M, N, K)
-    if tuple(vkey) != tuple(dkey):
-        vms, vtf = steady_gemm(be, vkey, M, N, K)
-        if vms < dms:
-            return vms, vtf, vkey
-    return dms, 2.0 * M * N * K / (dms * 1e-3) / 1e12, dkey
+def selected_and_model(be, prof_dict, M, N, K, verified):
+    """(key the runner launches, the cost model's first choice): the same key when verified is False."""
+    mkey = be.gemm.cost_model(prof_dict, M, N, K)
+    return (be.gemm.select_config(prof_dict, M, N, K) if verified else mkey), mkey
 
 
 def steady_vendor(be, M, N, K):
@@ -90,17 +85,16 @@ def steady_vendor(be, M, N, K):
 
 
 def square_rows(be, prof_dict, oracle=False, vendor=False, verified=True):
-    """Per size: the cost model's pick (Default) and the fastest of its first few candidates (Verified); oracle=True
-    adds the exhaustive per-shape search, vendor=True rocBLAS on the same operand layouts."""
+    """Per size: the runner's selection (and the cost model's first choice where it differs); oracle=True adds the
+    exhaustive per-shape search, vendor=True rocBLAS on the same operand layouts."""
     rows = []
     for s in S.BASELINE_SQUARE_SIZES:
-        key = be.gemm.cost_model(prof_dict, s, s, s)
+        key, mkey = selected_and_model(be, prof_dict, s, s, s, verified)
         ms, tflops = steady_gemm(be, key, s, s, s)
         row = {"M": s, "N": s, "K": s, "config": list(key), "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
-        if verified:
-            vms, vtf, vkey = steady_verified(be, prof_dict, key, ms, s, s, s)
-            row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
+        if tuple(mkey) != tuple(key):
+            row.update({"model_config": list(mkey), "model_us": round(steady_gemm(be, mkey, s, s, s)[0] * 1e3, 2)})
         if oracle:
             oms, otf, okey = steady_oracle(be, prof_dict, key, ms, s, s, s)
             row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2),
@@ -161,18 +155,18 @@ def conv_rows(be, prof_dict, vendor=False, oracle=False, verified=True):
     for shp in S.get_baseline_conv_shape_list():
         b, ic, h, w, oc, kh, kw, st, pd = shp
         M = b * ((h + 2 * pd - kh) // st + 1) * ((w + 2 * pd - kw) // st + 1)
-        key = be.conv.cost_model(prof_dict, M, oc, be.conv.gather_channels(ic) * kh * kw, be.conv.gather_channels(ic))
-        ms, tflops = be.conv_result(prof_dict, *shp)
+        mkey = be.conv.cost_model(prof_dict, M, oc, be.conv.gather_channels(ic) * kh * kw, be.conv.gather_channels(ic))
+        key = be.conv.select_config(prof_dict, *shp) if verified else mkey
+        ms = min(load(be.build.library_for_key(key)).bench_conv(*shp, warmup=10, iters=10)[1] for _ in range(3)) * 1e3
+        tflops = R.conv_flops(*shp) / (ms * 1e-3) / 1e12
         nbytes = R.conv_bytes(*shp, be.elem_bytes)
         rows.append({"shape": list(shp), "gemm_MNK": [M, oc, ic * kh * kw], "config": list(key), "us": round(ms * 1e3, 2),
                      "TFLOP/s": round(tflops, 2), "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4),
                      "GB/s": round(nbytes / (ms * 1e-3) / 1e9, 1),
                      "frac_hbm_peak": round(nbytes / (ms * 1e-3) / R.HBM_BYTES_PER_S, 4)})
-        if verified:
-            vms, vtf, vkey = be.conv_verified(prof_dict, *shp)
-            if vms >= ms:   # the Default configuration is the first candidate
-                vms, vkey = ms, key
-            rows[-1].update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2)})
+        if tuple(mkey) != tuple(key):
+            mms = min(load(be.build.library_for_key(mkey)).bench_conv(*shp, warmup=10, iters=10)[1] for _ in range(3)) * 1e3
+            rows[-1].update({"model_config": list(mkey), "model_us": round(mms * 1e3, 2)})
         if conv_oracle is not None:
             oms, otf, okey = conv_oracle(prof_dict, *shp)
             if oms >= ms:   # the Default configuration is one of the candidates
@@ -190,20 +184,19 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False, verified=True):
     latency, as the reference sums per-GEMM costs (benchmark_Ampere_FP16_model_level_LLM.py:16-27).  oracle=True adds
     the exhaustive per-shape search ("per-shape autotune"), vendor=True rocBLAS."""
     memo, rows = {}, []
-    totals = {"default": 0.0, "verified": 0.0, "oracle": 0.0, "rocblas": 0.0}
+    totals = {"default": 0.0, "model": 0.0, "oracle": 0.0, "rocblas": 0.0}
     total_flops = 0.0
     for (M, N, K) in S.get_baseline_bert_MNKList():
         if (M, N, K) not in memo:
-            dkey = be.gemm.cost_model(prof_dict, M, N, K)
+            dkey, mkey = selected_and_model(be, prof_dict, M, N, K, verified)
             ms, tflops = steady_gemm(be, dkey, M, N, K)
             row = {"M": M, "N": N, "K": K, "config": list(dkey),
                    "us": round(ms * 1e3, 2), "TFLOP/s": round(tflops, 2),
                    "frac_mfma_peak": round(tflops * 1e12 / be.peak, 4)}
-            times = {"default": ms}
-            if verified:
-                vms, vtf, vkey = steady_verified(be, prof_dict, dkey, ms, M, N, K)
-                row.update({"verified_config": list(vkey), "verified_us": round(vms * 1e3, 2), "verified_TFLOP/s": round(vtf, 2)})
-                times["verified"] = vms
+            times = {"default": ms, "model": ms}
+            if tuple(mkey) != tuple(dkey):
+                times["model"] = steady_gemm(be, mkey, M, N, K)[0]
+                row.update({"model_config": list(mkey), "model_us": round(times["model"] * 1e3, 2)})
             if oracle:
                 oms, otf, okey = steady_oracle(be, prof_dict, dkey, ms, M, N, K)
                 row.update({"oracle_config": list(okey), "oracle_us": round(oms * 1e3, 2), "oracle_TFLOP/s": round(otf, 2)})
@@ -220,8 +213,8 @@ def bert_rows(be, prof_dict, oracle=False, vendor=False, verified=True):
     tf = total_flops / (totals["default"] * 1e-3) / 1e12
     total = {"total_ms": round(totals["default"], 4), "TFLOP/s": round(tf, 2), "frac_mfma_peak": round(tf * 1e12 / be.peak, 4)}
     if verified:
-        vtf = total_flops / (totals["verified"] * 1e-3) / 1e12
-        total.update({"verified_total_ms": round(totals["verified"], 4), "verified_TFLOP/s": round(vtf, 2)})
+        mtf = total_flops / (totals["model"] * 1e-3) / 1e12
+        total.update({"model_total_ms": round(totals["model"], 4), "model_TFLOP/s": round(mtf, 2)})
     if oracle:
         otf = total_flops / (totals["oracle"] * 1e-3) / 1e12
         total.update({"oracle_total_ms": round(totals["oracle"], 4), "oracle_TFLOP/s": round(otf, 2),
@@ -260,7 +253,7 @@ if __name__ == "__main__":
     parser.add_argument("-b", "--backend", type=str, choices=MI355X_BACKENDS, default="MI355X_FP16")
     parser.add_argument("--oracle", action="store_true", help="square, bert, conv: also run the exhaustive per-shape search")
     parser.add_argument("--no-tiles", action="store_true", help="gemv: time the GEMV library only")
-    parser.add_argument("--no-verified", action="store_true", help="square, bert, conv: leave the Verified column out (Default launches only)")
+    parser.add_argument("--no-verified", action="store_true", help="square, bert, conv: run the cost model's first choice only (no candidates timed, no winners kept)")
     parser.add_argument("--vendor", action="store_true", help="conv: add MIOpen's time per layer; square, bert: add rocBLAS's")
     parser.add_argument("--json", action="store_true", help="one JSON object instead of the table")
     args = parser.parse_args()

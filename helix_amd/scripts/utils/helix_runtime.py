@@ -231,6 +231,7 @@ def read_prof_dict(backend):
 
 def write_prof_dict(backend, prof_dict):
     os.makedirs(os.path.dirname(prof_dict_path(backend)), exist_ok=True)
+    forget_winners(backend)   # winners were chosen among the old profile's rankings
     with open(prof_dict_path(backend), "w") as f:
         f.write(str(dict(prof_dict)))
     for attr, suffix in EXTRA_PROFILE_POINTS.items():
@@ -241,6 +242,66 @@ def write_prof_dict(backend, prof_dict):
                 f.write(str(dict(extra)))
         elif os.path.exists(path):
             os.remove(path)   # never pair a new profile with stale extra points
+
+
+# ---- per-problem winners ------------------------------------------------------------------------------------
+# The cost model ranks configurations from two profile points each; the first few of its ranking lie within a few
+# per cent of each other in prediction and 5 - 25 % apart on the device.  The runners therefore time the first few
+# candidates the first time they meet a problem (a few dozen launches) and keep the winner in a dict file beside the
+# profile, {problem tuple: configuration key}; later calls, in this process or another, go straight to it.  A new
+# profile (write_prof_dict) discards the file.  HELIX_SELECTION=model switches this off: the cost model alone
+# picks, as in the reference (scripts/Ampere_FP16/Ampere_FP16_gemm.py:433-446).
+def winners_path(backend):
+    return f"{root_path}/build/prof_dict/{backend}_winners.dict"
+
+
+def selection_mode():
+    mode = os.environ.get("HELIX_SELECTION", "tuned")
+    if mode not in ("tuned", "model"):
+        raise ValueError(f"HELIX_SELECTION={mode!r}: expected 'tuned' or 'model'")
+    return mode
+
+
+_winners = {}
+
+
+def read_winners(backend):
+    """The winners recorded for this backend ({} when there is no file yet); cached per process."""
+    if backend not in _winners:
+        path = winners_path(backend)
+        _winners[backend] = _read_dict_file(path) if os.path.exists(path) else {}
+    return _winners[backend]
+
+
+def store_winner(backend, problem, key):
+    winners = read_winners(backend)
+    winners[tuple(problem)] = tuple(key)
+    path = winners_path(backend)
+    os.makedirs(os.path.dirname(path), exist_ok=True)
+    tmp = f"{path}.{os.getpid()}.tmp"
+    with open(tmp, "w") as f:
+        f.write(str(winners))
+    os.replace(tmp, path)
+
+
+def forget_winners(backend):
+    _winners.pop(backend, None)
+    if os.path.exists(winners_path(backend)):
+        os.remove(winners_path(backend))
+
+
+def tuned_config(backend, problem, prof_dict, model_pick, verify):
+    """The configuration a runner launches for `problem`: the recorded winner if the profile still holds it, else
+    `verify()` (the fastest of the cost model's first candidates, timed now) which is then recorded; with
+    HELIX_SELECTION=model always `model_pick()`."""
+    if selection_mode() == "model":
+        return model_pick()
+    key = read_winners(backend).get(tuple(problem))
+    if key is not None and key in prof_dict:
+        return key
+    key = verify()
+    store_winner(backend, problem, key)
+    return key
 
 
 def reference_line(M, N, K, min_s, avg_s, max_s):

@@ -47,6 +47,7 @@ def saved_prof_dicts():
     yield directory
     shutil.rmtree(directory)
     shutil.move(backup, directory)
+    helix_runtime._winners.clear()      # winners recorded against the cheap profile are gone with its files
 
 
 def is_gemv_key(backend, k):

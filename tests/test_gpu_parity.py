@@ -81,17 +81,24 @@ def run_sgemm_f32(lib, A, B, workspace=True):
 
 FP16_CONFIGS = [(2, 256, 256, 128, 128, 64), (2, 256, 256, 64, 128, 64), (2, 128, 128, 64, 64, 128), (2, 64, 64, 32, 32, 64),
                 (2, 32, 32, 32, 32, 128), (2, 256, 64, 64, 32, 64), (2, 64, 256, 32, 128, 128), (2, 128, 256, 128, 64, 64),
-                (2, 128, 128, 64, 64, 64), (2, 256, 256, 128, 64, 64), (2, 64, 64, 32, 32, 128), (2, 32, 128, 32, 64, 64),
+                (2, 128, 128, 64, 64, 64), (2, 256, 256, 128, 64, 64), (2, 64, 64, 32, 32, 128), (2, 32, 128, 32, 32, 64),
                 # 48- and 96-column wave tiles (three and six MFMA tile columns per wave)
                 (2, 256, 192, 128, 96, 64), (2, 128, 96, 64, 48, 128), (2, 32, 48, 32, 48, 64), (2, 128, 192, 32, 96, 128),
                 (2, 256, 96, 64, 96, 64)]
+# split-K libraries are built for wave tiles of up to 32 x 64
+FP16_SPLITK_CONFIGS = [(2, 64, 64, 32, 32, 64), (2, 32, 32, 32, 32, 128), (2, 256, 64, 64, 32, 64), (2, 64, 256, 32, 64, 128),
+                       (2, 128, 128, 32, 64, 64), (2, 128, 128, 64, 32, 128), (2, 32, 128, 32, 64, 64), (2, 64, 192, 32, 48, 64),
+                       (2, 128, 96, 32, 48, 128), (2, 32, 48, 32, 48, 64), (2, 128, 64, 64, 32, 128)]
+
+
+def test_parity_configs_are_built_points():
+    assert set(FP16_CONFIGS) <= set(b16.iter_configs()) and set(FP16_SPLITK_CONFIGS) <= set(b16.iter_splitk_configs())
 
 
 # ---------------------------------------------------------------------------------------------
 # FP16 GEMM
 # ---------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("cfg", FP16_CONFIGS)
-@pytest.mark.parametrize("splitk", [0, 1])
+@pytest.mark.parametrize("splitk,cfg", [(0, c) for c in FP16_CONFIGS] + [(1, c) for c in FP16_SPLITK_CONFIGS])
 def test_gemm_f16_vs_oracle(cfg, splitk):
     lib = load(b16.kernel_library("gemm_splitK" if splitk else "gemm", *cfg))
     for (M, N, K) in [(256, 256, 256), (300, 200, 136), (1, 7, 8), (513, 1025, 72), (1024, 1024, 1024), (130, 260, 4096),
@@ -103,13 +110,13 @@ def test_gemm_f16_vs_oracle(cfg, splitk):
         assert normwise(got, want) < TOL16, (cfg, M, N, K)
 
 
-@pytest.mark.parametrize("cfg", FP16_CONFIGS[:4])
-def test_gemm_f16_integer_inputs_exact(cfg):
+@pytest.mark.parametrize("cfg,cfg_splitk", list(zip(FP16_CONFIGS[:4], FP16_SPLITK_CONFIGS[:4])))
+def test_gemm_f16_integer_inputs_exact(cfg, cfg_splitk):
     """Small integers: products and FP32 sums are exact, and the sums are kept below 2048 in magnitude so
     the FP16 result is exact too -- any wrong tile, edge or split-K index is an exact mismatch."""
     rng = np.random.default_rng(3)
     for splitk in (0, 1):
-        lib = load(b16.kernel_library("gemm_splitK" if splitk else "gemm", *cfg))
+        lib = load(b16.kernel_library("gemm_splitK", *cfg_splitk) if splitk else b16.kernel_library("gemm", *cfg))
         for (M, N, K) in [(257, 129, 200), (64, 500, 328)]:
             A = rng.integers(-2, 3, (M, K)).astype(np.float16)
             B = rng.integers(-2, 3, (K, N)).astype(np.float16)
@@ -214,7 +221,7 @@ def test_gemm_f16_rejects_bad_arguments():
     assert lib.gemm(p, p, C.data_ptr(), 0, 64, 64, 64, 64, 64, check=False) == HELIX_ERR_INVALID_VALUE
     with pytest.raises(HelixError):
         lib.gemm(p, p, C.data_ptr(), 64, 64, 60, 64, 64, 64)
-    sk = load(b16.kernel_library("gemm_splitK", 2, 128, 128, 64, 64, 64))
+    sk = load(b16.kernel_library("gemm_splitK", 2, 128, 128, 32, 64, 64))
     assert sk.workspace_bytes(64, 64, 64) == 2 * 64 * 64 * 4           # one K tile: the minimum 2-way split
     assert sk.workspace_bytes(64, 64, 4096) == 8 * 64 * 64 * 4         # one output tile, long K: 8-way
     assert sk.gemm(p, p, C.data_ptr(), 64, 64, 64, 64, 64, 64, 0, 0, check=False) == HELIX_ERR_WORKSPACE
@@ -319,8 +326,8 @@ CONV_GEOMS_ODD = [(2, 20, 20, 3, 16, 7, 7, 2, 3), (1, 9, 11, 1, 8, 5, 5, 2, 0), 
 
 
 @pytest.mark.parametrize("cfg", [(2, 128, 128, 64, 64, 64), (2, 64, 64, 32, 32, 64), (2, 256, 64, 64, 32, 64),
-                                 (2, 128, 64, 64, 32, 128), (2, 256, 256, 128, 64, 64), (2, 64, 128, 32, 64, 64),
-                                 (2, 128, 96, 64, 48, 128), (2, 64, 192, 32, 96, 64)])
+                                 (2, 128, 64, 64, 32, 128), (2, 256, 256, 128, 64, 64), (2, 64, 128, 32, 32, 64),
+                                 (2, 128, 96, 64, 48, 128), (2, 64, 192, 32, 48, 64)])
 def test_conv_f16_vs_oracle(cfg):
     lib = load(b16.kernel_library("gemm", *cfg))
     for (batch, H, W, IC, OC, kH, kW, stride, pad) in CONV_GEOMS + CONV_GEOMS_ODD:

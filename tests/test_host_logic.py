@@ -24,10 +24,11 @@ from MI355X_FP32 import MI355X_FP32_gemm as g32
 from MI355X_FP32 import MI355X_FP32_conv as c32
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-N_FP16_CONFIGS = 159   # points of the FP16 template space (tile x wave tile x BLOCK_K) that fit LDS and registers
-N_FP16_STAGES3 = 86    # of those, the points whose registers also hold a second staging set (K_STAGES = 3)
-N_FP16_SPLITK = 159    # every two-stage point also has a split-K variant
-N_FP16_DTL = 68        # points of the direct-to-LDS family: eight-wave tiles x (BLOCK_K, K_STAGES) in {32: 3, 4; 64: 2, 3}
+N_FP16_FIT = (159, 86, 68)   # points that fit the hardware: two-stage (each with a split-K twin), three-stage, direct-to-LDS
+N_FP16_CONFIGS = 106   # two-stage points the measured pruning keeps (workgroups of two waves are left out)
+N_FP16_STAGES3 = 81    # three-stage points kept (wave tiles of up to 64 rows)
+N_FP16_SPLITK = 62     # split-K libraries (wave tiles of up to 32 x 64)
+N_FP16_DTL = 2         # direct-to-LDS family: the 256 x 256 tile with two 64-column stages, both wave layouts
 
 
 # ---- enumeration ----------------------------------------------------------------------------------
@@ -44,6 +45,13 @@ def test_fp16_reference_validity_rules():
     assert not b16.is_valid_config(2, 2, 256, 256, 128, 128, 64, 4)   # two or three stages only
     assert b16.is_valid_config(2, 2, 128, 128, 64, 64, 64, 3)         # four waves, 64 accumulator registers each
     assert b16.is_valid_config(2, 4, 256, 256, 128, 64, 64, 2)        # 8 waves x 256 registers
+    # measured pruning on top of what fits: two-wave workgroups (two stages), 128-row wave tiles with three stages,
+    # split-K beyond 32 x 64 wave tiles
+    assert b16.fits_hardware(1, 2, 32, 128, 32, 64, 64, 2) and not b16.is_valid_config(1, 2, 32, 128, 32, 64, 64, 2)
+    assert b16.is_valid_config(1, 2, 32, 128, 32, 64, 64, 2, 1) and b16.is_valid_config(1, 2, 32, 128, 32, 64, 64, 3)
+    assert b16.fits_hardware(2, 2, 256, 64, 128, 32, 64, 3) and not b16.is_valid_config(2, 2, 256, 64, 128, 32, 64, 3)
+    assert b16.is_valid_config(2, 2, 128, 128, 64, 64, 64, 2) and not b16.is_valid_config(2, 2, 128, 128, 64, 64, 64, 2, 1)
+    assert b16.is_valid_config(2, 2, 128, 128, 32, 64, 64, 2, 1)
     assert b16.vgpr_estimate(256, 256, 128, 128, 64) == 256 + 80 + 64 + 16
     assert b16.vgpr_estimate(256, 256, 128, 64, 64) == 128 + 80 + 32 + 16      # exactly the 256 of two waves per SIMD
     assert b16.vgpr_estimate(128, 128, 64, 64, 64, 3) == 64 + 48 + 2 * 32 + 16   # two staging sets
@@ -60,9 +68,19 @@ def test_fp16_template_space():
         assert threads <= 512 and (br * bk // 8) % threads == 0 and (bc * bk // 8) % threads == 0
         assert b16.vgpr_estimate(br, bc, wr, wc, bk, st) <= 512 // ((threads // 64 + 3) // 4)
         if st == 3:      # every three-stage point is a two-stage point with room for the second staging set
-            assert (2, br, bc, wr, wc, bk) in cfgs
+            assert b16.fits_hardware(br // wr, bc // wc, br, bc, wr, wc, bk, 2) and wr <= 64
+        else:
+            assert (br // wr) * (bc // wc) != 2
+    splitk = list(b16.iter_splitk_configs())
+    assert len(splitk) == N_FP16_SPLITK and all(st == 2 and wr * wc <= 32 * 64 for (st, br, bc, wr, wc, bk) in splitk)
+    # the space before pruning
+    fit = [(st, rs, cs, wr, wc, bk) for st in (2, 3) for wr in b16.WAVE_TILE_LIST for wc in b16.WAVE_COLS_LIST
+           for rs in b16.BLOCK_SCALE_LIST for cs in b16.BLOCK_SCALE_LIST for bk in b16.BLOCK_K_LIST
+           if b16.fits_hardware(rs, cs, rs * wr, cs * wc, wr, wc, bk, st)]
+    assert (sum(1 for c in fit if c[0] == 2), sum(1 for c in fit if c[0] == 3)) == N_FP16_FIT[:2]
     assert (2, 256, 256, 128, 128, 64) in cfgs and (3, 256, 128, 64, 64, 64) in cfgs
     assert (3, 256, 256, 64, 128, 64) not in cfgs and (3, 256, 192, 64, 96, 64) not in cfgs
+    assert (2, 32, 128, 32, 64, 64) not in cfgs and (2, 32, 128, 32, 64, 64) in splitk
     keys = p16.all_keys()
     # a three-stage point whose GEMM kernel was recorded as spilling at build time is left out of the key list
     spilling3 = sum(1 for (st, br, bc, wr, wc, bk) in cfgs
@@ -76,25 +94,26 @@ def test_fp16_template_space():
 
 
 def test_fp16_direct_to_lds_space():
-    """The K_STAGES x DIRECT_TO_LDS axes: eight waves per workgroup, a ring of 2 .. 4 stages of 32 or 64 columns
-    within the 160 KiB of LDS, accumulators plus one K tile of fragments within 256 registers."""
+    """The K_STAGES x DIRECT_TO_LDS axes: eight waves per workgroup, a ring of stages within the 160 KiB of LDS,
+    accumulators plus one K tile of fragments within 256 registers; the build keeps the 256 x 256 tile with two
+    64-column stages."""
     cfgs = list(b16.iter_dtl_configs())
-    assert len(cfgs) == N_FP16_DTL and len(set(cfgs)) == N_FP16_DTL
+    assert cfgs == [(2, 256, 256, 64, 128, 64), (2, 256, 256, 128, 64, 64)] and len(cfgs) == N_FP16_DTL
     for (st, br, bc, wr, wc, bk) in cfgs:
         assert (br // wr) * (bc // wc) == 8 and br <= 256 and bc <= 256
         assert (bk, st) in b16.DTL_BK_STAGES_LIST and st * (br + bc) * bk * 2 + 64 <= 160 * 1024
         rows_per_copy = {32: 16, 64: 8}[bk]     # matrix rows one 1 KiB copy instruction fills
         assert (br // 4) % rows_per_copy == 0 and (bc // 4) % rows_per_copy == 0
         assert (bk // 32) * (wr // 16 + wc // 16) * 4 + (wr // 16) * (wc // 16) * 4 <= 236
-    assert (4, 256, 256, 128, 64, 32) in cfgs and (2, 256, 256, 128, 64, 64) in cfgs
-    assert (3, 256, 256, 128, 64, 64) not in cfgs       # three 64-column stages of a 256 x 256 tile exceed the LDS
-    assert b16.library_for_key((4, 256, 256, 128, 64, 0, 32, 1)).endswith("build/bin_fp16/libgemm_dtl_4_256_256_128_64_32.so")
-    src, out, defines = b16.compile_job("gemm_dtl", 4, 256, 256, 128, 64, 32)
-    assert src.endswith("src_template/MI355X_FP16/gemm_dtl.hip") and defines["K_STAGES"] == 4 and defines["BLOCK_K"] == 32
+    assert not b16.is_valid_dtl_config(2, 4, 256, 256, 128, 64, 64, 3)    # three 64-column stages of that tile exceed the LDS
+    assert not b16.is_valid_dtl_config(2, 4, 128, 256, 64, 64, 64, 2)     # other tiles: pruned
+    assert b16.library_for_key((2, 256, 256, 128, 64, 0, 64, 1)).endswith("build/bin_fp16/libgemm_dtl_2_256_256_128_64_64.so")
+    src, out, defines = b16.compile_job("gemm_dtl", 2, 256, 256, 128, 64, 64)
+    assert src.endswith("src_template/MI355X_FP16/gemm_dtl.hip") and defines["K_STAGES"] == 2 and defines["BLOCK_K"] == 64
     # no convolution entry: the conv cost model never picks the family
-    d = {(4, 256, 256, 128, 64, 0, 32, 1): 1e-9, (2, 128, 128, 64, 64, 0, 64): 1.0}
+    d = {(2, 256, 256, 128, 64, 0, 64, 1): 1e-9, (2, 128, 128, 64, 64, 0, 64): 1.0}
     assert c16.cost_model(d, 4096, 256, 576, 64) == (2, 128, 128, 64, 64, 0, 64)
-    assert g16.cost_model(d, 4096, 4096, 4096) == (4, 256, 256, 128, 64, 0, 32, 1)
+    assert g16.cost_model(d, 4096, 4096, 4096) == (2, 256, 256, 128, 64, 0, 64, 1)
 
 
 def test_fp16_library_names():
@@ -424,6 +443,61 @@ def test_prof_dict_roundtrip(tmp_path, monkeypatch):
     # a profile without them removes the stale files
     helix_runtime.write_prof_dict("MI355X_FP16", d)
     assert helix_runtime.read_prof_dict("MI355X_FP16").short == {}
+
+
+def test_winner_cache_and_selection_modes(tmp_path, monkeypatch):
+    """tuned_config: first meeting of a problem verifies and records, later ones read the record (also from a fresh
+    process: the file), a record the profile no longer holds is verified again, a new profile discards the file,
+    and HELIX_SELECTION=model asks the cost model alone."""
+    monkeypatch.setattr(helix_runtime, "root_path", str(tmp_path))
+    monkeypatch.setattr(helix_runtime, "_winners", {})
+    monkeypatch.delenv("HELIX_SELECTION", raising=False)
+    a, b, c = (2, 128, 128, 64, 64, 0, 64), (2, 64, 64, 64, 64, 0, 64), (3, 128, 128, 64, 64, 0, 64)
+    prof = {a: 1.0, b: 0.4}
+    calls = []
+
+    def verify(key):
+        def run():
+            calls.append(key)
+            return key
+        return run
+
+    problem = ("gemm", 512, 512, 512)
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(b)) == b and calls == [b]
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(a)) == b and calls == [b]
+    text = open(helix_runtime.winners_path("MI355X_FP16")).read()
+    assert text == str({problem: b}) and "\n" not in text
+    monkeypatch.setattr(helix_runtime, "_winners", {})                     # a fresh process reads the file
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(a)) == b and calls == [b]
+    assert helix_runtime.read_winners("MI355X_FP32") == {}                 # per backend
+    # the recorded configuration left the profile: verified again, record replaced
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, {a: 1.0, c: 0.9}, lambda: a, verify(c)) == c
+    assert calls == [b, c] and helix_runtime.read_winners("MI355X_FP16")[problem] == c
+    # the cost model alone
+    monkeypatch.setenv("HELIX_SELECTION", "model")
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(b)) == a and calls == [b, c]
+    monkeypatch.setenv("HELIX_SELECTION", "fastest")
+    with pytest.raises(ValueError):
+        helix_runtime.selection_mode()
+    monkeypatch.delenv("HELIX_SELECTION")
+    # a new profile discards the winners
+    helix_runtime.write_prof_dict("MI355X_FP16", prof)
+    assert not os.path.exists(helix_runtime.winners_path("MI355X_FP16")) and helix_runtime.read_winners("MI355X_FP16") == {}
+    # the dispatchers' select_config goes through it: problem keys per family, candidates from the model's ranking
+    monkeypatch.setattr(g16, "verified_config", lambda prof_dict, M, N, K, top=6: g16.ranked_configs(prof_dict, M, N, K, 2)[1])
+    picked = g16.select_config(prof, 4096, 4096, 4096)
+    assert picked == g16.ranked_configs(prof, 4096, 4096, 4096, 2)[1] != g16.cost_model(prof, 4096, 4096, 4096)
+    assert helix_runtime.read_winners("MI355X_FP16") == {("gemm", 4096, 4096, 4096): picked}
+    monkeypatch.setattr(c16, "verified_config", lambda prof_dict, *layer, top=6: b)
+    layer = (2, 64, 14, 14, 64, 3, 3, 1, 1)
+    assert c16.select_config(prof, *layer) == b
+    assert helix_runtime.read_winners("MI355X_FP16")[("conv",) + layer] == b
+    d32 = {b32.config_key(64, 64, 16, 32, 32): 1.0, b32.config_key(128, 64, 16, 32, 32): 1.7}
+    monkeypatch.setattr(g32, "verified_config", lambda prof_dict, M, N, K, top=6: b32.config_key(128, 64, 16, 32, 32))
+    assert g32.select_config(d32, 1024, 1024, 1024) == b32.config_key(128, 64, 16, 32, 32)
+    monkeypatch.setattr(c32, "verified_config", lambda prof_dict, *layer, top=6: b32.config_key(64, 64, 16, 32, 32))
+    assert c32.select_config(d32, *layer) == b32.config_key(64, 64, 16, 32, 32)
+    assert set(helix_runtime.read_winners("MI355X_FP32")) == {("gemm", 1024, 1024, 1024), ("conv",) + layer}
 
 
 def test_shape_lists():
