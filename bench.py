@@ -129,6 +129,26 @@ def engine_clock_mhz(run_for_s, work):
     return (int(statistics.median(samples)) if samples else None), per_call
 
 
+def mfma_ceiling():
+    """The matrix pipes with nothing else running (the MFMA-only loop of include/helix_probe.h, same instruction,
+    accumulators and waves per compute unit as the 256 x 256 x 64 GEMM tile), on seeded and on all-zero operands:
+    rate over about half a second each and the engine clock the driver reports meanwhile.  On seeded operands the
+    part runs against its power limit; this is the ceiling the GEMM rates above stand under."""
+    from utils.helix_runtime import probe_library
+    from utils.hip_ctypes import mfma_probe
+    path = probe_library("mfma_probe")
+    out = {}
+    for name, zeros in (("seeded", False), ("zeros", True)):
+        rates = []
+        clk, _ = engine_clock_mhz(0.5, lambda: rates.append(mfma_probe(path, zeros, warmup=1, launches=8, loops=500)[1]))
+        settled = rates[len(rates) // 2:]
+        out[name] = {"tflops": round(sum(settled) / len(settled), 1), "engine_clock_mhz": clk,
+                     "frac_datasheet_peak": round(sum(settled) / len(settled) * 1e12 / 2516.6e12, 4)}
+    out["how"] = ("MFMA-only loop (v_mfma_f32_16x16x32_f16, 8 waves per compute unit, operands in registers), "
+                  "second half of 0.5 s of launches each")
+    return out
+
+
 def cpu_baseline(budget_s=24.0):
     """The reference's x86_CPU path (restated in oracle/) on this machine's host cores: two-phase
     profile, tiling pick, then the packed / n-parallel schedule.  The headline sample is FP32 2048^3 (the
@@ -303,6 +323,7 @@ def main():
                                "vendor": round(flops / (per_v / batch) / 1e12, 2),
                                "how": "0.5 s of back-to-back launches each, wall clock"}
     del C2
+    out["mfma_only"] = mfma_ceiling()
     out["build_wall_s"] = build_times()
     if not args.no_gemv:
         out.update(other_configs())

@@ -28,7 +28,8 @@ GEMV_MFMA_MIN_M = 9                # MFMA_MIN_M of src_template/MI355X_FP16/gemv
 # for them no longer holds (measured: 661 x 768 x 3072 FP32, 103 us against 27 us)
 GEMV_MAX_ROWS = 16
 GEMV_SPLITK_EXTRA_S = 2e-6         # the K-partitioned GEMV library's reduction pass on a problem too small to need it
-SPLITK_REDUCE_LAUNCH_S = 4e-6      # the reduction kernel's launch, beyond what the profiled value already holds
+SPLITK_REDUCE_LAUNCH_S = 3e-6      # adding the partitions (the tail of the launch behind the last partial store, measured 3.3 us
+                                   # at eight partitions), beyond what the profiled value already holds
 ROUND_OVERLAP_S = 1e-6             # part of a round's fixed time that later rounds of one launch do not pay again
 
 

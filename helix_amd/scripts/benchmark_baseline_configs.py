@@ -116,12 +116,17 @@ def gemv_rows(be, prof_dict, rotate_bytes=1 << 30, tiles=True):
     nomfma = None if be.fp32 else load(be.build.kernel_library("gemv_nomfma"))
     tile_keys = [k for k in prof_dict if not be.is_gemv_key(k) and be.block_rows(k) == 32] if tiles else []
     rows = []
+    # what one launch costs when the kernel has next to nothing to do (same library, same back-to-back event timing,
+    # a 64 x 512 weight matrix): the part of every row's time that is launch and drain rather than streaming
+    floor = lib.bench(1, 64, 512, warmup=5, iters=50, outer=3, rotate_bytes=0)[0]
     for (K, N) in S.BASELINE_GEMV_KN:
         for M in S.BASELINE_GEMV_BATCHES:
             mn, _, _ = lib.bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)
             nbytes = R.gemm_bytes(M, N, K, be.elem_bytes)
             row = {"M": M, "K": K, "N": N, "us": round(mn * 1e6, 2), "GB/s": round(nbytes / mn / 1e9, 1),
-                   "frac_hbm_peak": round(nbytes / mn / R.HBM_BYTES_PER_S, 4)}
+                   "frac_hbm_peak": round(nbytes / mn / R.HBM_BYTES_PER_S, 4),
+                   "launch_floor_us": round(floor * 1e6, 2),
+                   "GB/s_above_floor": round(nbytes / max(mn - floor, 1e-9) / 1e9, 1)}
             if nomfma is not None and M >= 9:
                 mn_v = nomfma.bench(M, N, K, warmup=5, iters=50, outer=3, rotate_bytes=rotate_bytes)[0]
                 row["no_mfma_GB/s"] = round(nbytes / mn_v / 1e9, 1)

@@ -41,6 +41,16 @@ def bin_dir(precision):
     return f"{root_path}/build/bin_{precision}"
 
 
+def probe_library(name="mfma_probe"):
+    """Path of a measurement aid (include/helix_probe.h), built beside the template libraries."""
+    return f"{root_path}/build/bin_probe/lib{name}.so"
+
+
+def build_probes():
+    """Compiles the measurement aids of src_template/probe; returns the list of failures like compile_many."""
+    return compile_many([(os.path.join(SRC_ROOT, "probe", "mfma_probe.hip"), probe_library("mfma_probe"), {})])
+
+
 def prof_dict_path(backend):
     return f"{root_path}/build/prof_dict/{backend}_cost_model.dict"
 

@@ -142,6 +142,24 @@ class HelixLib:
         return mn.value, av.value, mx.value
 
 
+PROBE_SYMBOLS = ("helix_mfma_probe",)
+
+
+def mfma_probe(path, zero_operands=False, warmup=2, launches=10, loops=500):
+    """(seconds per launch, TFLOP/s) of the MFMA-only loop of include/helix_probe.h: what the matrix pipes sustain
+    with nothing else running, on seeded or on all-zero operands."""
+    if not os.path.exists(path):
+        raise FileNotFoundError(f"probe library {path} is not built; run __graft_entry__.build() first")
+    L = ctypes.CDLL(path)
+    L.helix_mfma_probe.argtypes = [_i, _i, _i, _i, _dp, _dp]
+    L.helix_mfma_probe.restype = _i
+    sec, flop = ctypes.c_double(), ctypes.c_double()
+    rc = L.helix_mfma_probe(1 if zero_operands else 0, warmup, launches, loops, ctypes.byref(sec), ctypes.byref(flop))
+    if rc != 0:
+        raise HelixError("helix_mfma_probe", rc)
+    return sec.value, flop.value / sec.value / 1e12
+
+
 def exported_symbols(path):
     """Names from ABI_SYMBOLS that `path` exports (no device needed: dlopen + dlsym only)."""
     L = ctypes.CDLL(path)

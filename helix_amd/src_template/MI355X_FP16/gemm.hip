@@ -18,9 +18,10 @@
 //                             their way through staging registers (2: one register set; 3: two, so that a load
 //                             has two tiles to land -- a few percent on mid-size tiles, where the registers allow
 //                             it)                                                  (reference K_STAGE)
-//   SPLIT_K                   1: each workgroup walks all of K.  > 1: K is partitioned over blockIdx.y into
-//                             2 .. SPLIT_K ranges, as many as it takes to give every compute unit a
-//                             workgroup (FP32 workspace + fixed-order reduction kernel)
+//   SPLIT_K                   1: each workgroup walks all of K.  > 1: K is partitioned into 2 .. SPLIT_K ranges, as
+//                             many as it takes to give every compute unit a workgroup (FP32 workspace; the
+//                             partitions of a tile are summed in order by the last of them to finish, inside
+//                             the launch, or by a reduction kernel where that is not available)
 //
 // Kernel structure
 //   * one wave64 computes (WAVE_ROWS/16) x (WAVE_COLS/16) v_mfma_f32_16x16x32_f16 tiles.  The 16x16x32
@@ -59,10 +60,6 @@ constexpr int RT = STAGES - 1;                 // K tiles in flight in staging r
 static_assert(LDS_BYTES <= 160 * 1024, "LDS budget of a gfx950 CU exceeded");
 
 __device__ __forceinline__ int swz_key(int row) { return (row / RP) & (KCH - 1); }
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, unsigned bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
 
 __device__ __forceinline__ intx4 buf_load16(__amdgpu_buffer_rsrc_t r, int voff) {
     // cache policy sc0 | sc1 (bits 0 and 4): a tile is read once per compute unit, so the loads go past the CU's
@@ -152,6 +149,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
     const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
 
     const TileRange tr = tile_range_of_workgroup(p);
+    if (tr.idle) return;
     const int m0 = tr.m0, n0 = tr.n0, k_begin = tr.k_begin, k_end = tr.k_end;
 
     // ---- per-thread copy geometry ---------------------------------------------------------------
@@ -466,7 +464,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             if (kt + u < ktiles) tile_step(kt + u, u & 1, st[(u + 1) % RT]);
     }
 
-    store_tile(acc, p, m0, n0, wave, wave_m, wave_n, lane, smem);
+    store_tile(acc, p, tr, tid, wave, wave_m, wave_n, lane, smem);
 }
 }  // namespace
 
@@ -511,11 +509,13 @@ inline int launch(const Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
     if (rc) return rc;
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
-    dim3 grid((unsigned)ntiles, (unsigned)p.splits, 1), block(NTHREADS, 1, 1);
-    hipLaunchKernelGGL(helix_gemm_f16_kernel<MODE>, grid, block, LDS_BYTES, s, p);
+    Params q = p;
+    const unsigned fused = fused_grid(q);   // K partitions summed inside the launch where that is available
+    dim3 grid(fused ? fused : (unsigned)ntiles, fused ? 1u : (unsigned)p.splits, 1), block(NTHREADS, 1, 1);
+    hipLaunchKernelGGL(helix_gemm_f16_kernel<MODE>, grid, block, LDS_BYTES, s, q);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    if (SPLITK > 1) {
+    if (SPLITK > 1 && !fused) {
         size_t total = (size_t)p.M * p.N;
         int blocks = (int)((total + 255) / 256);
         if (blocks > 8192) blocks = 8192;

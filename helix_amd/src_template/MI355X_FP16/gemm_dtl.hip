@@ -274,7 +274,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_dtl_kernel(const Para
     }
     if (grp == 0) phase_barrier();   // the barrier group 1 passes behind its last phase
 
-    store_tile(acc, p, m0, n0, wave, wave_m, wave_n, lane, smem);
+    store_tile(acc, p, tr, tid, wave, wave_m, wave_n, lane, smem);
 }
 
 }  // namespace

@@ -10,8 +10,12 @@
  *
  * Conventions
  *   - plain pointers and sizes only; device pointers come from hipMalloc (or any allocator layered
- *     on it); the library owns no persistent device memory and keeps no state besides a one-time
- *     function-attribute initialisation.
+ *     on it); the library allocates no device memory.  Its state is a one-time function-attribute
+ *     initialisation and what its device image holds: the scratch array of helix_gemm_static_scratch and, in
+ *     split-K libraries, 32 KiB of tile arrival counters (zero between launches) with the workgroup-id ->
+ *     XCD deal of the device, probed by the first split-K launch (one device synchronisation, so that first
+ *     launch must not happen under stream capture).  At most eight launches of one split-K library may be
+ *     in flight on one GPU at a time (they take turns on eight counter sets).
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
  *   - return value: 0 on success, a positive hipError_t value if the HIP runtime failed, or one of
  *     the HELIX_ERR_* codes.  Nothing throws, exits or prints.
@@ -60,7 +64,10 @@ HELIX_API int helix_info(char* json, int cap);
 
 /* Bytes of device scratch `helix_gemm` needs for this shape (0 unless the template splits K).
  * Replaces: nothing -- the reference's split-K accumulates with FP16 atomics into C
- * (src_template/Ampere_FP16/gemm_splitK.cu:495-506); here partial sums go through an FP32 workspace. */
+ * (src_template/Ampere_FP16/gemm_splitK.cu:495-506); here partial sums go through an FP32 workspace and are
+ * added in partition order, inside the launch by the last workgroup of a tile to finish or (environment
+ * HELIX_SPLITK_REDUCE=kernel, N not a multiple of 4, more than 1024 tiles, an irregular XCD deal) by a second
+ * kernel; both give the same bits. */
 HELIX_API size_t helix_workspace_bytes(int M, int N, int K);
 
 /* One GEMM / GEMV launch on `stream`.  lda/ldb/ldc are row strides in elements.

@@ -115,3 +115,15 @@ def test_helix_run_prints_the_reference_line():
     assert line.startswith("M N K =   1024   1024   1024, Time =")
     avg = float(line.split()[-8])        # the token the reference's profilers parse
     assert 1e-6 < avg < 1e-2 and line.endswith("Tflops")
+
+
+def test_mfma_probe_reports_a_plausible_ceiling():
+    """The MFMA-only loop: a rate between a fifth of and the whole datasheet peak, and all-zero operands (no
+    data-dependent power draw) not slower than seeded ones."""
+    from utils.helix_runtime import probe_library
+    from utils.hip_ctypes import mfma_probe
+    path = probe_library("mfma_probe")
+    seeded = max(mfma_probe(path, False, warmup=2, launches=10, loops=300)[1] for _ in range(3))
+    zeros = max(mfma_probe(path, True, warmup=2, launches=10, loops=300)[1] for _ in range(3))
+    assert 500.0 < seeded < 2516.6 * 1.02 and 500.0 < zeros < 2516.6 * 1.02, (seeded, zeros)
+    assert zeros > 0.97 * seeded, (seeded, zeros)

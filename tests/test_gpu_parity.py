@@ -208,6 +208,56 @@ def test_gemm_f16_full_size_properties(key, full_size_operands):
     assert (dC2.float() - 2 * dC.float()).abs().max().item() <= 2.0 ** -23
 
 
+SPLITK_PATH_SCRIPT = r"""
+import sys, numpy as np, torch
+sys.path.insert(0, sys.argv[2]); sys.path.insert(0, sys.argv[3]); sys.path.insert(0, sys.argv[4])
+from utils import seeded_inputs
+from utils.helix_runtime import load
+from MI355X_FP16 import build_MI355X_FP16 as b16
+from gpu_helpers import run_gemm_f16, run_conv
+out = {}
+for ci, cfg in enumerate([(2, 64, 64, 32, 32, 128), (2, 128, 128, 32, 64, 64), (2, 32, 128, 32, 32, 64)]):
+    lib = load(b16.kernel_library("gemm_splitK", *cfg))
+    for (M, N, K) in [(196, 512, 4608), (130, 260, 4096), (8, 4096, 1024), (1000, 72, 520)]:
+        A, B = seeded_inputs.gemm_operands(M, N, K, np.float16)
+        out[f"g{ci}_{M}_{N}_{K}"] = run_gemm_f16(lib, A, B)
+    x, w = seeded_inputs.conv_operands(4, 256, 7, 7, 128, 3, 3)
+    out[f"c{ci}"] = run_conv(lib, x, w, 1, 1, torch.float16)
+np.savez(sys.argv[1], **out)
+"""
+
+
+def test_splitk_in_launch_sum_and_reduction_kernel_give_identical_bits(tmp_path):
+    """Split-K libraries add a tile's partitions inside the launch (the last workgroup of the tile to finish, all on
+    one XCD) or, with HELIX_SPLITK_REDUCE=kernel, in a second kernel: same partials, same order of FP32 additions, so
+    the FP16 results are bit-identical; both are within tolerance of the oracle."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    args = [os.path.join(root, "helix_amd", "scripts"), os.path.join(root, "tests"), root]
+    outs = {}
+    for mode in ("in_launch", "kernel"):
+        env = dict(os.environ, HELIX_DEBUG="1")
+        env.pop("HELIX_SPLITK_REDUCE", None)
+        if mode == "kernel":
+            env["HELIX_SPLITK_REDUCE"] = "kernel"
+        path = str(tmp_path / f"{mode}.npz")
+        run = subprocess.run([sys.executable, "-c", SPLITK_PATH_SCRIPT, path] + args, capture_output=True, text=True,
+                             env=env, cwd=root, timeout=300)
+        assert run.returncode == 0, run.stderr[-2000:]
+        # the in-launch path announces the workgroup id -> XCC_ID deal it found; the kernel path never probes
+        assert ("deals workgroup ids 0..7 to XCC_IDs" in run.stderr) == (mode == "in_launch"), run.stderr[-500:]
+        outs[mode] = dict(np.load(path))
+    assert outs["in_launch"].keys() == outs["kernel"].keys() and len(outs["kernel"]) == 15
+    for name, got in outs["in_launch"].items():
+        assert not np.isnan(got).any(), name
+        assert np.array_equal(got.view(np.uint16), outs["kernel"][name].view(np.uint16)), name
+    A, B = seeded_inputs.gemm_operands(196, 512, 4608, np.float16)
+    assert normwise(outs["in_launch"]["g0_196_512_4608"], O.hgemm_f32acc(A, B)) < TOL16
+    x, w = seeded_inputs.conv_operands(4, 256, 7, 7, 128, 3, 3)
+    assert normwise(outs["in_launch"]["c1"], O.conv2d_nhwc(x, w, 1, 1)) < TOL16
+
+
 def test_gemm_f16_rejects_bad_arguments():
     lib = load(b16.kernel_library("gemm", 2, 128, 128, 64, 64, 64))
     A = torch.zeros((64, 64), dtype=torch.float16, device="cuda:0")

@@ -617,6 +617,22 @@ def test_libraries_export_only_the_abi():
         assert want <= names, path
 
 
+def test_probe_library_exports_what_its_header_declares():
+    text = open(os.path.join(ROOT, "include", "helix_probe.h")).read()
+    declared = sorted(set(re.findall(r"^HELIX_PROBE_API\s+int\s+(helix_\w+)\s*\(", text, flags=re.M)))
+    assert declared == sorted(hip_ctypes.PROBE_SYMBOLS)
+    path = helix_runtime.probe_library("mfma_probe")
+    assert path.endswith("build/bin_probe/libmfma_probe.so")
+    if not os.path.exists(path):
+        pytest.skip("probe library is not built (run __graft_entry__.build())")
+    out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+    names = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    assert set(declared) <= names
+    assert not {n for n in names - set(declared) if not n.startswith("__hip_cuid_") and n != "_ZSt19piecewise_construct"}
+    with pytest.raises(FileNotFoundError):
+        hip_ctypes.mfma_probe(path + ".missing")
+
+
 def test_all_expected_libraries_are_built():
     if not _built_libraries():
         pytest.skip("kernel libraries are not built (run __graft_entry__.build())")
