@@ -113,8 +113,10 @@ def cost_model(prof_dict, M, N, K):
 # "Verified" selection: the cost model ranks, the device decides among the first few.  Predictions of the leading
 # configurations lie within a few per cent of each other while their measured times differ by 5 - 25 %; timing
 # VERIFY_TOP of them once per shape (a handful of launches, against hundreds for the exhaustive search) recovers
-# most of that (measured over 30 convolution layers: picked / fastest 1.07 -> 1.03 with four candidates, 1.02 with six).
-VERIFY_TOP = 6
+# most of that (measured over 30 convolution layers: picked / fastest 1.07 -> 1.03 with four candidates, 1.02 with six,
+# 1.015 with eight).  The runners keep the winner per problem (utils.helix_runtime.tuned_config), so the candidates of
+# a problem are timed once per profile: twelve of them.
+VERIFY_TOP = 12
 
 
 def ranked_configs(prof_dict, M, N, K, top=VERIFY_TOP):

@@ -134,7 +134,7 @@ def cost_model(prof_dict, M, N, K):
 
 # "Verified" selection: the cost model ranks, the device decides among the first few (the leading predictions lie
 # within a per cent of each other for configurations that measure 5 - 10 % apart).
-VERIFY_TOP = 6
+VERIFY_TOP = 12
 
 
 def ranked_configs(prof_dict, M, N, K, top=VERIFY_TOP):

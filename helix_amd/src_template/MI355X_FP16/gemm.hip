@@ -464,7 +464,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_kernel(const Params p
             if (kt + u < ktiles) tile_step(kt + u, u & 1, st[(u + 1) % RT]);
     }
 
-    store_tile(acc, p, tr, tid, wave, wave_m, wave_n, lane, smem);
+    store_tile<LDS_BYTES>(acc, p, tr, tid, wave, wave_m, wave_n, lane, smem);
 }
 }  // namespace
 
@@ -510,12 +510,11 @@ inline int launch(const Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
     Params q = p;
-    const unsigned fused = fused_grid(q);   // K partitions summed inside the launch where that is available
-    dim3 grid(fused ? fused : (unsigned)ntiles, fused ? 1u : (unsigned)p.splits, 1), block(NTHREADS, 1, 1);
+    const dim3 grid = launch_grid(q), block(NTHREADS, 1, 1);   // K partitions added inside the launch where available
     hipLaunchKernelGGL(helix_gemm_f16_kernel<MODE>, grid, block, LDS_BYTES, s, q);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    if (SPLITK > 1 && !fused) {
+    if (SPLITK > 1 && !q.plan.fused) {
         size_t total = (size_t)p.M * p.N;
         int blocks = (int)((total + 255) / 256);
         if (blocks > 8192) blocks = 8192;

@@ -274,7 +274,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_gemm_f16_dtl_kernel(const Para
     }
     if (grp == 0) phase_barrier();   // the barrier group 1 passes behind its last phase
 
-    store_tile(acc, p, tr, tid, wave, wave_m, wave_n, lane, smem);
+    store_tile<LDS_BYTES>(acc, p, tr, tid, wave, wave_m, wave_n, lane, smem);
 }
 
 }  // namespace
@@ -329,11 +329,11 @@ inline int gemm(const void* A, const void* B, void* C, int M, int N, int K, int 
     if (rc) return rc;
     const long long ntiles = (long long)p.tiles_m * p.tiles_n;
     if (ntiles > 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
-    dim3 grid((unsigned)ntiles, (unsigned)p.splits, 1), block(NTHREADS, 1, 1);
+    const dim3 grid = launch_grid(p), block(NTHREADS, 1, 1);   // K partitions added inside the launch where available
     hipLaunchKernelGGL(helix_gemm_f16_dtl_kernel<>, grid, block, LDS_BYTES, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    if (SPLITK > 1) {
+    if (SPLITK > 1 && !p.plan.fused) {
         size_t total = (size_t)M * N;
         int blocks = (int)((total + 255) / 256);
         if (blocks > 8192) blocks = 8192;

@@ -14,11 +14,12 @@
 // Compile-time parameters: BM x BN workgroup tile, BK (K extent of one LDS stage), WAVE_M x WAVE_N, K_GROUPS
 // (waves per wave tile, each taking BK / K_GROUPS of every K tile; 1 unless the configuration is a K-group one).
 //
-// K partitions: a problem is split along K over blockIdx.y, up to 8 ways, when that shortens the launch: few
-// tiles and a long K (compute units idle), or a tile count that leaves the last round of workgroups mostly
-// empty (split_factor below); partial sums go to the caller's workspace (helix_workspace_bytes) and a second
-// kernel adds them in partition order.  Without the workspace the problem runs unpartitioned.  The
-// reference's FP32 template has no K partition.
+// K partitions: a problem is split along K, up to 8 ways, when that shortens the launch: few tiles and a long K
+// (compute units idle), or a tile count that leaves the last round of workgroups mostly empty (split_factor
+// below); partial sums go to the caller's workspace (helix_workspace_bytes) and are added in partition order by
+// the last workgroup of a tile to finish (all partitions of a tile run on one XCD, common/helix_splitk.h) or,
+// where that is not available (K-group configurations among them), by a second kernel; same bits either way.
+// Without the workspace the problem runs unpartitioned.  The reference's FP32 template has no K partition.
 //
 // LDS layout: A stage is [BK][BM + 32] floats, B stage [BK][BN + 32]; a fragment read takes lanes 0-31
 // from row k and lanes 32-63 from row k+1, and the 32-float row padding puts the two half-waves on
@@ -32,6 +33,7 @@
 #include "helix_abi.h"
 #include "helix_im2col.h"
 #include "helix_fastdiv.h"
+#include "helix_splitk.h"
 
 #ifndef BM
 #define BM 128
@@ -120,8 +122,9 @@ struct Params {
     int tiles_m, tiles_n;
     unsigned a_bytes;
     float* ws;       // splits > 1: [splits][M][N] partial sums
-    int splits;      // K partitions of this launch (grid.y)
+    int splits;      // K partitions of this launch
     int k_per;       // K extent of one partition, a multiple of BK
+    helix_splitk::Plan plan;   // how the partitions of a tile are added
     ConvGeom g;
 };
 
@@ -148,14 +151,11 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     const int wave_kg = wave / WAVES_MN, wave_mn = wave % WAVES_MN;
     const int wave_m = wave_mn / WAVES_N, wave_n = wave_mn % WAVES_N;
 
-    // workgroup id -> tile: undo the round-robin deal over the 8 XCDs, then walk groups of tile rows
-    const int ntiles = p.tiles_m * p.tiles_n;
-    int pid = blockIdx.x;
-    {
-        const int per = ntiles / 8, rem = ntiles % 8;
-        const int xcd = pid % 8, slot = pid / 8;
-        pid = xcd * per + (xcd < rem ? xcd : rem) + slot;
-    }
+    // workgroup id -> tile number (the round-robin deal over the 8 XCDs undone: each XCD is given a compact run of
+    // tile numbers) and K partition, then walk groups of tile rows
+    const helix_splitk::Unit unit = helix_splitk::unit_of_workgroup(p.plan, p.tiles_m * p.tiles_n, p.splits);
+    if (unit.idle) return;
+    const int pid = unit.tile;
     const int group_tiles = GROUP_ROWS * p.tiles_n;
     const int first_m = (pid / group_tiles) * GROUP_ROWS;
     const int gsize = (p.tiles_m - first_m) < GROUP_ROWS ? (p.tiles_m - first_m) : GROUP_ROWS;
@@ -164,7 +164,7 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     // K range of this workgroup
-    const int k_lo = (int)blockIdx.y * p.k_per;
+    const int k_lo = unit.split * p.k_per;
     const int k_hi = (k_lo + p.k_per) < p.K ? (k_lo + p.k_per) : p.K;
 
     constexpr int NA = CONV ? AC_ITERS : A_ITERS;
@@ -404,11 +404,19 @@ __global__ __launch_bounds__(NTHREADS) void helix_sgemm_f32_kernel(const Params 
             for (int v = 0; v < 16; v++) {
                 const int row = m0 + wave_m * WAVE_M + i * 32 + (v / 4) * 8 + row_l + (v % 4);
                 if (row < p.M && col < p.N) {
-                    if (p.splits > 1) p.ws[((size_t)blockIdx.y * p.M + row) * p.N + col] = acc[i][j][v];
+                    if (p.splits > 1) p.ws[((size_t)unit.split * p.M + row) * p.N + col] = acc[i][j][v];
                     else __builtin_nontemporal_store(acc[i][j][v], &p.C[(size_t)row * p.ldc + col]);   // not read again by this launch
                 }
             }
         }
+    }
+    if (KG == 1 && p.splits > 1 && p.plan.fused) {           // else helix_sgemm_splitk_reduce_kernel adds the partials
+        // loads in flight while adding: what the main loop's registers already allow (32 where LDS keeps the kernel to
+        // two waves per SIMD, 16 from 64 accumulator registers per lane on, else 8)
+        constexpr bool ROOMY = ((160 * 1024) / LDS_BYTES) * NWAVES <= 8;
+        constexpr int LOADS = ROOMY ? 32 : (TM * TN * 16 >= 64 ? 16 : 8);
+        helix_splitk::sum_partitions_if_last<float, BM, BN, NTHREADS, 8, LOADS>(
+            p.plan, p.ws, p.C, p.M, p.N, p.ldc, p.splits, pid, m0, n0, tid, (unsigned char*)smem);
     }
 }
 
@@ -519,11 +527,14 @@ inline int launch(Params& p, void* ws, size_t ws_bytes, hipStream_t s) {
     const int ktiles = (p.K + BK - 1) / BK;
     p.k_per = ((ktiles + p.splits - 1) / p.splits) * BK;
     p.ws = (float*)ws;
-    hipLaunchKernelGGL(helix_sgemm_f32_kernel<CONV>, dim3((unsigned)ntiles, (unsigned)p.splits), dim3(NTHREADS),
-                       LDS_BYTES, s, p);
+    // partitions added inside the launch where that is available (one-dimensional grid), else by the second kernel
+    p.plan = helix_splitk::Plan{0, 0u, nullptr};
+    const unsigned fused = KG == 1 ? helix_splitk::plan_launch(p.plan, ntiles, p.splits, p.M, p.N) : 0u;
+    const dim3 grid = fused ? dim3(fused, 1, 1) : dim3((unsigned)ntiles, (unsigned)p.splits, 1);
+    hipLaunchKernelGGL(helix_sgemm_f32_kernel<CONV>, grid, dim3(NTHREADS), LDS_BYTES, s, p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
-    if (p.splits > 1) {
+    if (p.splits > 1 && !fused) {
         const size_t total = (size_t)p.M * p.N;
         int blocks = (int)((total + 255) / 256);
         if (blocks > 8192) blocks = 8192;

@@ -88,7 +88,7 @@ def test_candidate_performance_curve(prof16, capsys):
     best_id, best_config, rows = curve.get_all_candidate_performance(prof16, M, N, K)
     assert len(rows) == len(prof16) and 1 <= best_id <= len(rows) and best_config in prof16
     measured = [t for (_, _, t) in rows if t is not None]
-    assert len(measured) > 300 and max(measured) > 1.0
+    assert len(measured) > 200 and max(measured) > 1.0
     picked = rows[best_id - 1][2]
     assert picked is not None and picked > 0.6 * max(measured), (picked, max(measured))
     out = capsys.readouterr().out

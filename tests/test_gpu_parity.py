@@ -223,12 +223,21 @@ for ci, cfg in enumerate([(2, 64, 64, 32, 32, 128), (2, 128, 128, 32, 64, 64), (
         out[f"g{ci}_{M}_{N}_{K}"] = run_gemm_f16(lib, A, B)
     x, w = seeded_inputs.conv_operands(4, 256, 7, 7, 128, 3, 3)
     out[f"c{ci}"] = run_conv(lib, x, w, 1, 1, torch.float16)
+from MI355X_FP32 import build_MI355X_FP32 as b32
+from gpu_helpers import run_sgemm_f32
+for ci, cfg in enumerate([(64, 64, 32, 32, 32), (128, 128, 16, 32, 64)]):
+    lib = load(b32.sgemm_library(*cfg))
+    for (M, N, K) in [(300, 200, 4096), (100, 96, 1000), (661, 768, 3072)]:
+        assert lib.workspace_bytes(M, N, K) > 0
+        A = seeded_inputs.uniform_pm1((M, K), seeded_inputs.SEED_A)
+        B = seeded_inputs.uniform_pm1((K, N), seeded_inputs.SEED_B)
+        out[f"s{ci}_{M}_{N}_{K}"] = run_sgemm_f32(lib, A, B)
 np.savez(sys.argv[1], **out)
 """
 
 
 def test_splitk_in_launch_sum_and_reduction_kernel_give_identical_bits(tmp_path):
-    """Split-K libraries add a tile's partitions inside the launch (the last workgroup of the tile to finish, all on
+    """Split-K libraries (FP16) and K-partitioned launches (FP32) add a tile's partitions inside the launch (the last workgroup of the tile to finish, all on
     one XCD) or, with HELIX_SPLITK_REDUCE=kernel, in a second kernel: same partials, same order of FP32 additions, so
     the FP16 results are bit-identical; both are within tolerance of the oracle."""
     import subprocess
@@ -248,10 +257,14 @@ def test_splitk_in_launch_sum_and_reduction_kernel_give_identical_bits(tmp_path)
         # the in-launch path announces the workgroup id -> XCC_ID deal it found; the kernel path never probes
         assert ("deals workgroup ids 0..7 to XCC_IDs" in run.stderr) == (mode == "in_launch"), run.stderr[-500:]
         outs[mode] = dict(np.load(path))
-    assert outs["in_launch"].keys() == outs["kernel"].keys() and len(outs["kernel"]) == 15
+    assert outs["in_launch"].keys() == outs["kernel"].keys() and len(outs["kernel"]) == 15 + 6
     for name, got in outs["in_launch"].items():
         assert not np.isnan(got).any(), name
-        assert np.array_equal(got.view(np.uint16), outs["kernel"][name].view(np.uint16)), name
+        bits = np.uint16 if got.dtype == np.float16 else np.uint32
+        assert np.array_equal(got.view(bits), outs["kernel"][name].view(bits)), name
+    A32 = seeded_inputs.uniform_pm1((300, 4096), seeded_inputs.SEED_A)
+    B32 = seeded_inputs.uniform_pm1((4096, 200), seeded_inputs.SEED_B)
+    assert normwise(outs["in_launch"]["s0_300_200_4096"], O.sgemm_seqk(A32, B32)) < TOL32
     A, B = seeded_inputs.gemm_operands(196, 512, 4608, np.float16)
     assert normwise(outs["in_launch"]["g0_196_512_4608"], O.hgemm_f32acc(A, B)) < TOL16
     x, w = seeded_inputs.conv_operands(4, 256, 7, 7, 128, 3, 3)
