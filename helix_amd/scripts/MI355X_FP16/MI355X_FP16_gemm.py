@@ -27,6 +27,13 @@ GEMV_MFMA_MIN_M = 9                # MFMA_MIN_M of src_template/MI355X_FP16/gemv
 # which reads them once per BLOCK_ROWS rows, is the better streamer, and the per-round share the model assumes
 # for them no longer holds (measured: 661 x 768 x 3072 FP32, 103 us against 27 us)
 GEMV_MAX_ROWS = 16
+# Timing loops (the reference's and these) launch again and again on the same buffers, so weights that fit the 256 MB
+# memory-side cache stream from it: measured on M = 1 and 2, 33 MB of weights take 0.45 of their share of the profiled
+# (268 MB, HBM-bound) launch, 75 MB 0.66, 100 MB 0.72, 150 MB 0.83
+GEMV_RESIDENT_BYTES = 32e6
+GEMV_STREAMED_BYTES = 200e6
+GEMV_RESIDENT_SHARE = 0.45
+GEMV_DOT_MACS_PER_S = 18e12        # v_dot2 variant, measured at 8 rows on 4096 x 4096 and 9216 x 4096 weights
 GEMV_SPLITK_EXTRA_S = 2e-6         # the K-partitioned GEMV library's reduction pass on a problem too small to need it
 SPLITK_REDUCE_LAUNCH_S = 3e-6      # adding the partitions (the tail of the launch behind the last partial store, measured 3.3 us
                                    # at eight partitions), beyond what the profiled value already holds
@@ -43,6 +50,16 @@ def split_factor(k, M, N, K):
     ktiles = math.ceil(K / k[6])
     s = min(NUM_CU // max(tiles, 1), SPLITK_MAX, ktiles // 2)
     return max(s, 2)
+
+
+def resident_share(weight_bytes):
+    """Share of the profiled (HBM-bound) streaming time that weights of this size take in a timing loop."""
+    if weight_bytes <= GEMV_RESIDENT_BYTES:
+        return GEMV_RESIDENT_SHARE
+    if weight_bytes >= GEMV_STREAMED_BYTES:
+        return 1.0
+    ramp = (weight_bytes - GEMV_RESIDENT_BYTES) / (GEMV_STREAMED_BYTES - GEMV_RESIDENT_BYTES)
+    return GEMV_RESIDENT_SHARE + (1.0 - GEMV_RESIDENT_SHARE) * ramp
 
 
 def round_time(v, v_short, K):
@@ -66,13 +83,20 @@ def config_cost(k, v, M, N, K, v_short=None):
         # weight-streaming kernel: HBM-bound, so a partial round costs its share of a round (no
         # quantisation), never less than a launch; the streamed operand is the larger of M and N
         small, big = (M, N) if M <= N else (N, M)
-        if small > GEMV_MAX_ROWS:
+        if small > GEMV_MAX_ROWS or small > k[1]:
+            # the three rows of a family are one library profiled at 1, 4 and 16 activation rows: a row describes
+            # problems of up to its own row count (the reference's ceil(M / rows) passes, Ampere_FP16_gemm.py:420,
+            # would charge a pass per row tile for what the kernel does in one)
             return float("inf")
-        num_block = math.ceil(small / k[1]) * math.ceil(big / k[2])
+        num_block = math.ceil(big / k[2])
         floor = GEMV_LAUNCH_FLOOR_S if small < GEMV_MFMA_MIN_M else GEMV_MFMA_FLOOR_S
+        k_walk = max(K, 512)
         # the profiled launch holds one launch's fixed time, which does not scale with the problem
-        stream = max(v - GEMV_LAUNCH_FLOOR_S, 0.0)
-        cost = max(GEMV_LAUNCH_FLOOR_S + num_block / NUM_CU * stream * max(K, 512) / PROFILE_K, floor)
+        stream = max(v - GEMV_LAUNCH_FLOOR_S, 0.0) * num_block / NUM_CU * k_walk / PROFILE_K
+        stream *= resident_share(big * k_walk * 2)
+        # below the MFMA variant every activation row costs a dot-product instruction per weight pair
+        dots = small * big * k_walk / GEMV_DOT_MACS_PER_S if small < GEMV_MFMA_MIN_M else 0.0
+        cost = floor + max(stream, dots)
         return cost + (GEMV_SPLITK_EXTRA_S if k[5] == 1 else 0.0)
     splits = split_factor(k, M, N, K)
     num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * splits

@@ -176,15 +176,25 @@ def test_fp16_cost_model_hand_cases():
     assert c1 < c0
     assert g16.config_cost((2, 128, 128, 64, 64, 1, 64), 1.0, 4096 * 4, 4096, K) > \
         g16.config_cost((2, 128, 128, 64, 64, 0, 64), 1.0, 4096 * 4, 4096, K) * 0.99
-    # GEMV rows: blocks = ceil(small / row tile) * ceil(big / 128), proportional share of a 256-block round
+    # GEMV rows: a row describes problems of up to its own row count; blocks = ceil(big / 128), a proportional share of
+    # a 256-block round of the part of the profiled launch beyond one launch's fixed time (GEMV_LAUNCH_FLOOR_S)
     gemv = (0, 4, 128, 0, 0, 0, 0)
-    # of the part of the profiled launch beyond one launch's fixed time (GEMV_LAUNCH_FLOOR_S)
     fixed, stream = g16.GEMV_LAUNCH_FLOOR_S, 2.56e-3 - g16.GEMV_LAUNCH_FLOOR_S
+    assert g16.resident_share(128 * 256 * K * 2) == 1.0            # 268 MB of weights: streamed from HBM
     assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 256, K) == pytest.approx(2.56e-3)
-    assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 128, K) == pytest.approx(fixed + stream / 2)
     assert g16.config_cost(gemv, 2.56e-3, 128 * 256, 3, K) == pytest.approx(2.56e-3)      # operands swap
-    assert g16.config_cost(gemv, 2.56e-3, 16, 128 * 256, K) == pytest.approx(fixed + 4 * stream)
-    assert g16.config_cost(gemv, 1e-9, 1, 128, 512) == g16.GEMV_LAUNCH_FLOOR_S
+    assert g16.config_cost(gemv, 2.56e-3, 5, 128 * 256, K) == float("inf")                # the 16-row profile row's case
+    assert g16.config_cost((0, 16, 128, 0, 0, 0, 0), 2.56e-3, 17, 128 * 256, K) == float("inf")
+    # weights that stay in the memory-side cache between launches take a smaller share of the profiled stream
+    half = 128 * 128 * K * 2
+    share = g16.resident_share(half)
+    assert g16.GEMV_RESIDENT_SHARE < share < 1.0
+    assert share == pytest.approx(0.45 + 0.55 * (half - 32e6) / (200e6 - 32e6))
+    assert g16.config_cost(gemv, 2.56e-3, 4, 128 * 128, K) == pytest.approx(fixed + share * stream / 2)
+    assert g16.resident_share(1e6) == g16.GEMV_RESIDENT_SHARE
+    # the dot-product variant is bound by its instruction rate when the stream is short
+    assert g16.config_cost(gemv, 4e-6, 4, 128 * 256, K) == pytest.approx(fixed + 4 * 128 * 256 * K / g16.GEMV_DOT_MACS_PER_S)
+    assert g16.config_cost(gemv, 1e-9, 1, 128, 512) == pytest.approx(g16.GEMV_LAUNCH_FLOOR_S, rel=2e-3)  # never less than a launch
     # conv never selects a GEMV row
     d2 = dict(d)
     d2[gemv] = 1e-12
@@ -290,8 +300,9 @@ def test_fp16_cost_model_two_point_profile():
     # GEMV rows: 9 or more activation rows run the K-partitioned MFMA variant (higher floor); the split-K
     # GEMV library pays its reduction
     assert g16.config_cost((0, 16, 128, 0, 0, 0, 0), 1e-9, 13, 128, 512) == g16.GEMV_MFMA_FLOOR_S
+    dots = 4 * 128 * 512 / g16.GEMV_DOT_MACS_PER_S
     assert g16.config_cost((0, 16, 128, 0, 0, 1, 0), 1e-9, 4, 128, 512) == \
-        pytest.approx(g16.GEMV_LAUNCH_FLOOR_S + g16.GEMV_SPLITK_EXTRA_S)
+        pytest.approx(g16.GEMV_LAUNCH_FLOOR_S + dots + g16.GEMV_SPLITK_EXTRA_S)
 
 
 def test_fp32_split_factor_rule():
