@@ -26,7 +26,7 @@ SIZE = 8192
 # the counter values.  A configuration without a counted run reports null: the figure cannot be measured from
 # inside this process.
 MEASURED_TRAFFIC = {
-    (2, 256, 256, 64, 128, 0, 64): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
+    (2, 256, 256, 64, 128, 0, 64): (1.748e9, "profiles/gemm_f16_8192_pmc.md"),
     (2, 256, 256, 128, 64, 0, 64): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
     (2, 256, 256, 128, 128, 0, 64): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
     (2, 256, 256, 64, 128, 0, 64, 1): (1.745e9, "profiles/gemm_f16_8192_pmc.md"),
