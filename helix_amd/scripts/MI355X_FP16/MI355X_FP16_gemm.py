@@ -33,7 +33,7 @@ GEMV_MAX_ROWS = 16
 GEMV_RESIDENT_BYTES = 32e6
 GEMV_STREAMED_BYTES = 200e6
 GEMV_RESIDENT_SHARE = 0.45
-GEMV_DOT_MACS_PER_S = 18e12        # v_dot2 variant, measured at 8 rows on 4096 x 4096 and 9216 x 4096 weights
+GEMV_WIDE_STREAM_ROWS = 4          # activation-row tiles up to this many rows keep 8 KiB of loads in flight per wave
 GEMV_SPLITK_EXTRA_S = 2e-6         # the K-partitioned GEMV library's reduction pass on a problem too small to need it
 SPLITK_REDUCE_LAUNCH_S = 3e-6      # adding the partitions (the tail of the launch behind the last partial store, measured 3.3 us
                                    # at eight partitions), beyond what the profiled value already holds
@@ -93,10 +93,11 @@ def config_cost(k, v, M, N, K, v_short=None):
         k_walk = max(K, 512)
         # the profiled launch holds one launch's fixed time, which does not scale with the problem
         stream = max(v - GEMV_LAUNCH_FLOOR_S, 0.0) * num_block / NUM_CU * k_walk / PROFILE_K
-        stream *= resident_share(big * k_walk * 2)
-        # below the MFMA variant every activation row costs a dot-product instruction per weight pair
-        dots = small * big * k_walk / GEMV_DOT_MACS_PER_S if small < GEMV_MFMA_MIN_M else 0.0
-        cost = floor + max(stream, dots)
+        # the eight-row tile of the dot-product variant keeps half as many loads in flight and streams cache-resident
+        # weights no faster than cold ones (4096 x 4096 at 8 rows 10.3 us against 5.4 us at one row)
+        if small <= GEMV_WIDE_STREAM_ROWS or small >= GEMV_MFMA_MIN_M:
+            stream *= resident_share(big * k_walk * 2)
+        cost = floor + stream
         return cost + (GEMV_SPLITK_EXTRA_S if k[5] == 1 else 0.0)
     splits = split_factor(k, M, N, K)
     num_block = math.ceil(M / k[1]) * math.ceil(N / k[2]) * splits
