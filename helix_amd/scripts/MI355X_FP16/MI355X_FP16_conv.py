@@ -11,7 +11,7 @@ repack + GEMM), all on one stream and timed as one.
 import math
 import os
 
-from utils.helix_runtime import load, kernel_resources, tuned_config
+from utils.helix_runtime import load, kernel_resources, tuned_config, fastest_of
 from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, is_dtl_key
 from MI355X_FP16.MI355X_FP16_gemm import short_value, config_cost, VERIFY_TOP
 
@@ -112,21 +112,16 @@ def ranked_configs(prof_dict, M, N, K, IC=None, top=VERIFY_TOP):
 
 
 def verified_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, top=VERIFY_TOP):
-    """The fastest of the cost model's first `top` configurations on this layer, each timed with 2 + 5 launches."""
+    """The fastest of the cost model's first `top` configurations on this layer (utils.helix_runtime.fastest_of:
+    2 + 5 launches each, the leaders timed again)."""
     M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
     ICg = gather_channels(input_channel)
-    timed, last_error = [], None
-    for k in ranked_configs(prof_dict, M, output_channel, ICg * kH * kW, ICg, top):
-        try:
-            _, avg, _ = load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride,
-                                                            pad, warmup=2, iters=5)
-        except Exception as e:     # a candidate that cannot run this layer is skipped, as the profile skips it
-            last_error = e
-            continue
-        timed.append((avg, k))
-    if not timed:
-        raise RuntimeError(f"none of the {top} ranked configurations could run this layer") from last_error
-    return min(timed)[1]
+
+    def time_config(k, warmup, iters):
+        return load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
+                                                   warmup=warmup, iters=iters)[1]
+
+    return fastest_of(ranked_configs(prof_dict, M, output_channel, ICg * kH * kW, ICg, top), time_config, "this layer")
 
 
 def get_MI355X_FP16_conv_Verified_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,

@@ -7,7 +7,7 @@ has no counterpart: the only backend value is "hip".
 import math
 import os
 
-from utils.helix_runtime import load, tuned_config
+from utils.helix_runtime import load, tuned_config, fastest_of
 from utils.roofline import NUM_CU, HBM_BYTES_PER_S, gemm_bytes
 from MI355X_FP16.build_MI355X_FP16 import library_for_key, kernel_library, SPLITK_MAX
 from MI355X_FP16.profile_MI355X_FP16 import PROFILE_K, PROFILE_K_SHORT
@@ -168,16 +168,10 @@ def run_config(k, M, N, K, warmup=10, iters=10, outer=1):
 
 
 def verified_config(prof_dict, M, N, K, top=VERIFY_TOP):
-    """The fastest of the cost model's first `top` configurations on this problem, each timed with 2 + 5 launches."""
-    timed, last_error = [], None
-    for k in ranked_configs(prof_dict, M, N, K, top):
-        try:
-            timed.append((run_config(k, M, N, K, warmup=2, iters=5), k))
-        except Exception as e:     # a candidate that cannot run this shape is skipped, as the profile skips it
-            last_error = e
-    if not timed:
-        raise RuntimeError(f"none of the {top} ranked configurations could run {M}x{N}x{K}") from last_error
-    return min(timed)[1]
+    """The fastest of the cost model's first `top` configurations on this problem (utils.helix_runtime.fastest_of:
+    2 + 5 launches each, the leaders timed again)."""
+    return fastest_of(ranked_configs(prof_dict, M, N, K, top),
+                      lambda k, warmup, iters: run_config(k, M, N, K, warmup=warmup, iters=iters), f"{M}x{N}x{K}")
 
 
 def select_config(prof_dict, M, N, K):

@@ -5,7 +5,7 @@ point pads the channels to a multiple of 4 in its workspace first (IC = 1: FP32 
 import math
 import os
 
-from utils.helix_runtime import load, tuned_config
+from utils.helix_runtime import load, tuned_config, fastest_of
 from MI355X_FP32.build_MI355X_FP32 import library_for_key, kernel_library
 from MI355X_FP32.MI355X_FP32_gemm import config_cost, extra_points, VERIFY_TOP
 
@@ -52,20 +52,16 @@ def ranked_configs(prof_dict, M, N, K, top=VERIFY_TOP):
 
 
 def verified_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad, top=VERIFY_TOP):
-    """The fastest of the cost model's first `top` configurations on this layer, each timed with 2 + 5 launches."""
+    """The fastest of the cost model's first `top` configurations on this layer (utils.helix_runtime.fastest_of:
+    2 + 5 launches each, the leaders timed again)."""
     M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
-    timed, last_error = [], None
-    for k in ranked_configs(prof_dict, M, output_channel, gather_channels(input_channel) * kH * kW, top):
-        try:
-            _, avg, _ = load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride,
-                                                            pad, warmup=2, iters=5)
-        except Exception as e:     # a candidate that cannot run this layer is skipped, as the profile skips it
-            last_error = e
-            continue
-        timed.append((avg, k))
-    if not timed:
-        raise RuntimeError(f"none of the {top} ranked configurations could run this layer") from last_error
-    return min(timed)[1]
+
+    def time_config(k, warmup, iters):
+        return load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
+                                                   warmup=warmup, iters=iters)[1]
+
+    return fastest_of(ranked_configs(prof_dict, M, output_channel, gather_channels(input_channel) * kH * kW, top),
+                      time_config, "this layer")
 
 
 def get_MI355X_FP32_conv_Verified_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,

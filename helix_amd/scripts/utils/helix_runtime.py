@@ -300,6 +300,35 @@ def forget_winners(backend):
         os.remove(winners_path(backend))
 
 
+SETTLE_FINALISTS = 4        # candidates timed a second time ...
+SETTLE_WITHIN = 1.10        # ... those within this factor of the fastest of the first pass
+
+
+def fastest_of(keys, time_config, what):
+    """The fastest of `keys` on the device.  time_config(key, warmup, iters) -> mean seconds per launch, raising for a
+    configuration that cannot run the problem (skipped, as the profile skips it).  First pass: 2 + 5 launches each.  The
+    leaders of that pass lie within its noise of each other (a 5-launch mean right behind another kernel moves by
+    5 - 10 % with the engine clock), so up to SETTLE_FINALISTS of them within SETTLE_WITHIN of the fastest are timed
+    again, two rounds of 5 + 20 launches in turn, and the smallest mean decides."""
+    timed, last_error = [], None
+    for k in keys:
+        try:
+            timed.append((time_config(k, 2, 5), k))
+        except Exception as e:
+            last_error = e
+    if not timed:
+        raise RuntimeError(f"none of the {len(keys)} ranked configurations could run {what}") from last_error
+    timed.sort(key=lambda tk: tk[0])
+    finalists = [k for t, k in timed[:SETTLE_FINALISTS] if t <= timed[0][0] * SETTLE_WITHIN]
+    if len(finalists) == 1:
+        return finalists[0]
+    best = {k: float("inf") for k in finalists}
+    for _ in range(2):
+        for k in finalists:
+            best[k] = min(best[k], time_config(k, 5, 20))
+    return min(finalists, key=lambda k: best[k])
+
+
 def tuned_config(backend, problem, prof_dict, model_pick, verify):
     """The configuration a runner launches for `problem`: the recorded winner if the profile still holds it, else
     `verify()` (the fastest of the cost model's first candidates, timed now) which is then recorded; with

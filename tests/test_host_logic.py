@@ -457,6 +457,32 @@ def test_prof_dict_roundtrip(tmp_path, monkeypatch):
     assert helix_runtime.read_prof_dict("MI355X_FP16").short == {}
 
 
+def test_fastest_of_times_the_leaders_again():
+    """First pass 2 + 5 launches each; the candidates within 10 % of its fastest (at most four) are timed again, two
+    rounds of 5 + 20 in turn, and the smallest of those means decides; a candidate that cannot run is skipped."""
+    calls = []
+    first = {"a": 1.00, "b": 0.97, "c": 2.0, "e": 1.05, "f": 1.06, "g": 1.065}
+    second = {"a": [0.95, 0.99], "b": [1.0, 0.96], "e": [1.2, 1.2], "f": [1.3, 1.3]}
+
+    def time_config(k, warmup, iters):
+        calls.append((k, warmup, iters))
+        if k == "d":
+            raise RuntimeError("cannot run")
+        if iters == 5:
+            return first[k]
+        return second[k].pop(0)
+
+    assert helix_runtime.fastest_of(["a", "b", "c", "d", "e", "f", "g"], time_config, "p") == "a"
+    assert calls[:7] == [(k, 2, 5) for k in "abcdefg"]
+    # b, a, e, f in first-pass order, twice round; c (beyond 10 %), g (fifth) and d (failed) are not timed again
+    assert calls[7:] == [(k, 5, 20) for k in "baef"] * 2
+    calls.clear()
+    assert helix_runtime.fastest_of(["c", "a"], time_config, "p") == "a" and calls == [("c", 2, 5), ("a", 2, 5)]
+    with pytest.raises(RuntimeError, match="none of the 1 ranked configurations could run p") as err:
+        helix_runtime.fastest_of(["d"], time_config, "p")
+    assert "cannot run" in str(err.value.__cause__)
+
+
 def test_winner_cache_and_selection_modes(tmp_path, monkeypatch):
     """tuned_config: first meeting of a problem verifies and records, later ones read the record (also from a fresh
     process: the file), a record the profile no longer holds is verified again, a new profile discards the file,
