@@ -4,7 +4,8 @@ Mirrors scripts/Ampere_FP16/Ampere_FP16_conv.py:420-446: the conv is mapped to G
 M = batch*OH*OW, N = OC, K = IC*kH*kW (:432-434), the GEMM cost model picks the configuration, and
 the cost is measured.  The reference runs an im2col executable plus the GEMM executable and adds the
 two times (:437-445); here the selected configuration's library gathers the A tile on the fly (one
-kernel, one time) when IC is a multiple of 8; otherwise the same entry point first pads the channels of
+kernel, one time) when IC is a multiple of 8 (a 1 x 1 filter with stride 1 and no padding gathers nothing and runs
+as the plain GEMM on the activations as they lie); otherwise the same entry point first pads the channels of
 activations and weights to a multiple of 8 in its workspace (or, for IC = 1 and 2, runs im2col + weight
 repack + GEMM), all on one stream and timed as one.
 """
@@ -49,7 +50,15 @@ def resident_workgroups(k):
     return max(1, min(LDS_BYTES_PER_CU // lds, WAVES_PER_CU // waves, 8))
 
 
-def conv_config_cost(k, v, M, N, K, v_short=None, IC=None):
+def is_pointwise(kH, kW, stride, pad):
+    """A 1 x 1 filter walked pixel by pixel: the library runs such a layer as the plain GEMM on the activations as they
+    lie (gemm.hip, conv2d), so no gather term applies and no gather kernel's registers matter."""
+    return kH == 1 and kW == 1 and stride == 1 and pad == 0
+
+
+def conv_config_cost(k, v, M, N, K, v_short=None, IC=None, pointwise=False):
+    if pointwise:
+        return config_cost(k, v, M, N, K, v_short)
     short = math.ceil(K / k[6]) <= SHORT_K_TILES
     per_column = SHORT_K_GATHER_COST_PER_TILE_COLUMN if short else GATHER_COST_PER_TILE_COLUMN
     cost = config_cost(k, v, M, N, K, v_short) * (1.0 + per_column * math.ceil(N / k[2]))
@@ -82,31 +91,31 @@ def conv_kernel_scratch(k, IC=None):
     return 0
 
 
-def cost_model(prof_dict, M, N, K, IC=None):
+def cost_model(prof_dict, M, N, K, IC=None, pointwise=False):
     """GEMM cost model restricted to the MFMA configurations with a conv entry (gemm.hip's), with the
-    gather terms above; IC is the channel count the kernel walks (gather_channels)."""
+    gather terms above; IC is the channel count the kernel walks (gather_channels); pointwise: is_pointwise()."""
     min_cost = float("inf")
     best_config = (1, 1, 1, 1, 1, 0, 32)
     for k, v in prof_dict.items():
         if k[0] == 0 or is_dtl_key(k):      # neither the GEMV nor the direct-to-LDS libraries have a conv entry
             continue
-        if conv_kernel_scratch(k, IC) > 0:  # a spilling gather is never the fastest one
+        if not pointwise and conv_kernel_scratch(k, IC) > 0:  # a spilling gather is never the fastest one
             continue
-        cost = conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC)
+        cost = conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC, pointwise)
         if min_cost > cost:
             min_cost = cost
             best_config = k
     return best_config
 
 
-def ranked_configs(prof_dict, M, N, K, IC=None, top=VERIFY_TOP):
+def ranked_configs(prof_dict, M, N, K, IC=None, top=VERIFY_TOP, pointwise=False):
     """The `top` convolution-capable configurations with the lowest predicted cost, best first; cost_model returns
     the first of them."""
     cand = []
     for k, v in prof_dict.items():
-        if k[0] == 0 or is_dtl_key(k) or conv_kernel_scratch(k, IC) > 0:
+        if k[0] == 0 or is_dtl_key(k) or (not pointwise and conv_kernel_scratch(k, IC) > 0):
             continue
-        cand.append((conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC), k))
+        cand.append((conv_config_cost(k, v, M, N, K, short_value(prof_dict, k), IC, pointwise), k))
     cand.sort()
     return [k for _, k in cand[:top]]
 
@@ -121,7 +130,9 @@ def verified_config(prof_dict, batch, input_channel, H, W, output_channel, kH, k
         return load(library_for_key(k)).bench_conv(batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
                                                    warmup=warmup, iters=iters)[1]
 
-    return fastest_of(ranked_configs(prof_dict, M, output_channel, ICg * kH * kW, ICg, top), time_config, "this layer")
+    return fastest_of(ranked_configs(prof_dict, M, output_channel, ICg * kH * kW, ICg, top,
+                                     is_pointwise(kH, kW, stride, pad) and input_channel % GATHER_CHUNK == 0),
+                      time_config, "this layer")
 
 
 def get_MI355X_FP16_conv_Verified_result(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad,
@@ -136,15 +147,21 @@ def get_MI355X_FP16_conv_Verified_result(prof_dict, batch, input_channel, H, W, 
     return cost * 1e3, flops / 1e12 / cost, best
 
 
+def layer_cost_model(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
+    """cost_model on the GEMM extents of a layer (Ampere_FP16_conv.py:432-435)."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    ICg = gather_channels(input_channel)
+    return cost_model(prof_dict, M, output_channel, ICg * kH * kW, ICg,
+                      is_pointwise(kH, kW, stride, pad) and input_channel % GATHER_CHUNK == 0)
+
+
 def select_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
     """The configuration the runner launches for this layer: the cost model's ranking, settled on the device the first
     time the layer is met and remembered beside the profile (utils.helix_runtime.tuned_config); the cost model's
     first choice alone with HELIX_SELECTION=model."""
-    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
-    ICg = gather_channels(input_channel)
     layer = (batch, input_channel, H, W, output_channel, kH, kW, stride, pad)
     return tuned_config("MI355X_FP16", ("conv",) + layer, prof_dict,
-                        lambda: cost_model(prof_dict, M, output_channel, ICg * kH * kW, ICg),
+                        lambda: layer_cost_model(prof_dict, *layer),
                         lambda: verified_config(prof_dict, *layer))
 
 

@@ -76,14 +76,19 @@ def get_MI355X_FP32_conv_Verified_result(prof_dict, batch, input_channel, H, W, 
     return cost * 1e3, flops / 1e12 / cost, best
 
 
+def layer_cost_model(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
+    """cost_model on the GEMM extents of a layer (Ampere_FP32_conv.py's mapping)."""
+    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
+    return cost_model(prof_dict, M, output_channel, gather_channels(input_channel) * kH * kW)
+
+
 def select_config(prof_dict, batch, input_channel, H, W, output_channel, kH, kW, stride, pad):
     """The configuration the runner launches for this layer: the cost model's ranking, settled on the device the first
     time the layer is met and remembered beside the profile (utils.helix_runtime.tuned_config); the cost model's
     first choice alone with HELIX_SELECTION=model."""
-    M = batch * ((H + 2 * pad - kH) // stride + 1) * ((W + 2 * pad - kW) // stride + 1)
     layer = (batch, input_channel, H, W, output_channel, kH, kW, stride, pad)
     return tuned_config("MI355X_FP32", ("conv",) + layer, prof_dict,
-                        lambda: cost_model(prof_dict, M, output_channel, gather_channels(input_channel) * kH * kW),
+                        lambda: layer_cost_model(prof_dict, *layer),
                         lambda: verified_config(prof_dict, *layer))
 
 

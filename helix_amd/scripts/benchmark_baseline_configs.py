@@ -160,7 +160,7 @@ def conv_rows(be, prof_dict, vendor=False, oracle=False, verified=True):
     for shp in S.get_baseline_conv_shape_list():
         b, ic, h, w, oc, kh, kw, st, pd = shp
         M = b * ((h + 2 * pd - kh) // st + 1) * ((w + 2 * pd - kw) // st + 1)
-        mkey = be.conv.cost_model(prof_dict, M, oc, be.conv.gather_channels(ic) * kh * kw, be.conv.gather_channels(ic))
+        mkey = be.conv.layer_cost_model(prof_dict, *shp)
         key = be.conv.select_config(prof_dict, *shp) if verified else mkey
         ms = min(load(be.build.library_for_key(key)).bench_conv(*shp, warmup=10, iters=10)[1] for _ in range(3)) * 1e3
         tflops = R.conv_flops(*shp) / (ms * 1e-3) / 1e12

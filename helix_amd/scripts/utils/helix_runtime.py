@@ -258,8 +258,9 @@ def write_prof_dict(backend, prof_dict):
 # The cost model ranks configurations from two profile points each; the first few of its ranking lie within a few
 # per cent of each other in prediction and 5 - 25 % apart on the device.  The runners therefore time the first few
 # candidates the first time they meet a problem (a few dozen launches) and keep the winner in a dict file beside the
-# profile, {problem tuple: configuration key}; later calls, in this process or another, go straight to it.  A new
-# profile (write_prof_dict) discards the file.  HELIX_SELECTION=model switches this off: the cost model alone
+# profile, {problem tuple: configuration key} plus one entry that names the profile by its contents; later calls under
+# the same profile, in this process or another, go straight to it; under any other profile the record starts afresh.  A
+# new profile file (write_prof_dict) discards the file.  HELIX_SELECTION=model switches this off: the cost model alone
 # picks, as in the reference (scripts/Ampere_FP16/Ampere_FP16_gemm.py:433-446).
 def winners_path(backend):
     return f"{root_path}/build/prof_dict/{backend}_winners.dict"
@@ -273,18 +274,30 @@ def selection_mode():
 
 
 _winners = {}
+PROFILE_TAG = ("profile",)     # the entry of a winners file that names the profile its winners were ranked and timed under
 
 
-def read_winners(backend):
-    """The winners recorded for this backend ({} when there is no file yet); cached per process."""
+def profile_fingerprint(prof_dict):
+    """Names a profile by its contents: winners recorded under one profile are not handed out under another (a profile
+    of other libraries or another machine state, a hand-made dict in a test)."""
+    import hashlib
+    return hashlib.md5(repr(sorted(prof_dict.items())).encode()).hexdigest()
+
+
+def read_winners(backend, prof_dict):
+    """The winners recorded for this backend under this profile ({} when there is no file yet or the file belongs to
+    another profile); the file is read once per process."""
     if backend not in _winners:
         path = winners_path(backend)
         _winners[backend] = _read_dict_file(path) if os.path.exists(path) else {}
+    tag = profile_fingerprint(prof_dict)
+    if _winners[backend].get(PROFILE_TAG) != tag:
+        _winners[backend] = {PROFILE_TAG: tag}
     return _winners[backend]
 
 
-def store_winner(backend, problem, key):
-    winners = read_winners(backend)
+def store_winner(backend, problem, key, prof_dict):
+    winners = read_winners(backend, prof_dict)
     winners[tuple(problem)] = tuple(key)
     path = winners_path(backend)
     os.makedirs(os.path.dirname(path), exist_ok=True)
@@ -335,11 +348,11 @@ def tuned_config(backend, problem, prof_dict, model_pick, verify):
     HELIX_SELECTION=model always `model_pick()`."""
     if selection_mode() == "model":
         return model_pick()
-    key = read_winners(backend).get(tuple(problem))
+    key = read_winners(backend, prof_dict).get(tuple(problem))
     if key is not None and key in prof_dict:
         return key
     key = verify()
-    store_winner(backend, problem, key)
+    store_winner(backend, problem, key, prof_dict)
     return key
 
 

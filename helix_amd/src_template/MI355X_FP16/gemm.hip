@@ -625,6 +625,10 @@ inline int conv2d(const void* x, const void* w, void* y, int batch, int H, int W
     const long long xbytes = (long long)batch * H * W * IC * 2;
     if (M > 0x7fffffffLL || K > 0x7fffffffLL || xbytes >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
     if ((long long)BN * K * 2 >= 0x7fffffffLL) return HELIX_ERR_INVALID_VALUE;
+    // a 1 x 1 filter walked pixel by pixel gathers nothing: the activations as they lie are the A operand (rows =
+    // pixels, K = IC), so the layer is the plain GEMM and runs without the gather's index arithmetic
+    if (kH == 1 && kW == 1 && stride == 1 && pad == 0)
+        return gemm(x, w, y, (int)M, OC, IC, IC, IC, OC, ws, ws_bytes, s);
     Params p{};
     p.A = (const half_t*)x; p.B = (const half_t*)w; p.C = (half_t*)y; p.ws = (float*)ws;
     p.M = (int)M; p.N = OC; p.K = (int)K; p.lda = 0; p.ldb = (int)K; p.ldc = OC;

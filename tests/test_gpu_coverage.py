@@ -77,14 +77,18 @@ def _int_conv_cases(rng, dtype, channel_counts):
         exact = O.conv2d_nhwc(x.astype(np.float32), w.astype(np.float32), stride, pad)
         assert np.abs(exact).max() < 2048
         out.append((x, w, stride, pad, exact))
+    # a 1 x 1 filter walked pixel by pixel (the FP16 libraries run it as the plain GEMM on the activations as they lie)
+    x = rng.integers(-1, 2, (3, 5, 7, 72)).astype(dtype)
+    w = rng.integers(-1, 2, (40, 1, 1, 72)).astype(dtype)
+    out.append((x, w, 1, 0, O.conv2d_nhwc(x.astype(np.float32), w.astype(np.float32), 1, 0)))
     return out
 
 
 @pytest.mark.parametrize("keys", _chunks(FP16_TILE_KEYS), ids=lambda ks: f"{ks[0]}..")
 def test_every_fp16_library_integer_exact(keys):
-    """Per configuration: two ragged GEMMs (a narrow first K tile, a split-K partition with a remainder) and four
+    """Per configuration: two ragged GEMMs (a narrow first K tile, a split-K partition with a remainder) and five
     convolutions -- IC = 128 and 64 (a K tile inside one filter tap when IC is a multiple of BLOCK_K), IC = 8
-    (the general gather), IC = 3 (channel-padded copies in the workspace)."""
+    (the general gather), IC = 3 (channel-padded copies in the workspace), and a 1 x 1 stride-1 layer."""
     rng = np.random.default_rng(100)
     gemms = _int_gemm_cases(rng, np.float16)
     convs = _int_conv_cases(rng, np.float16, (128, 64, 8, 3))

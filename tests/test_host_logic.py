@@ -457,6 +457,29 @@ def test_prof_dict_roundtrip(tmp_path, monkeypatch):
     assert helix_runtime.read_prof_dict("MI355X_FP16").short == {}
 
 
+def test_pointwise_layers_are_ranked_as_the_gemm_they_run_as():
+    """1 x 1, stride 1, no padding, channels on the gather chunk: the FP16 library runs the layer through its GEMM
+    entry, so the convolution model adds no gather term and does not look at the gather kernels' registers."""
+    assert c16.is_pointwise(1, 1, 1, 0) and not c16.is_pointwise(1, 1, 2, 0) and not c16.is_pointwise(3, 3, 1, 1)
+    assert not c16.is_pointwise(1, 1, 1, 1)
+    k = (2, 128, 128, 64, 64, 0, 64)
+    assert c16.conv_config_cost(k, 60e-6, 100352, 256, 64, 8e-6, 64, pointwise=True) == \
+        g16.config_cost(k, 60e-6, 100352, 256, 64, 8e-6)
+    assert c16.conv_config_cost(k, 60e-6, 100352, 256, 64, 8e-6, 64) > g16.config_cost(k, 60e-6, 100352, 256, 64, 8e-6)
+    d = {(2, 128, 128, 64, 64, 0, 64): 600e-6, (2, 64, 64, 32, 32, 0, 64): 220e-6, (0, 1, 128, 0, 0, 0, 0): 1e-9,
+         (2, 256, 256, 64, 128, 0, 64, 1): 1e-9}    # values large enough that no floor of the model binds
+    layer = (32, 64, 56, 56, 256, 1, 1, 1, 0)
+    M = 32 * 56 * 56
+    pick = c16.layer_cost_model(d, *layer)
+    assert pick == c16.cost_model(d, M, 256, 64, 64, pointwise=True) and pick[0] != 0 and not b16.is_dtl_key(pick)
+    assert pick == min((k for k in d if k[0] and not b16.is_dtl_key(k)), key=lambda k: g16.config_cost(k, d[k], M, 256, 64))
+    assert c16.ranked_configs(d, M, 256, 64, 64, 12, pointwise=True)[0] == pick
+    # stride 2 or channels off the chunk: the gather model
+    assert c16.layer_cost_model(d, 32, 64, 56, 56, 256, 1, 1, 2, 0) == c16.cost_model(d, 32 * 28 * 28, 256, 64, 64)
+    assert c16.layer_cost_model(d, 32, 3, 56, 56, 256, 1, 1, 1, 0) == c16.cost_model(d, M, 256, 8, 8)
+    assert c32.layer_cost_model({b32.config_key(64, 64, 16, 32, 32): 1.0}, *layer) == b32.config_key(64, 64, 16, 32, 32)
+
+
 def test_fastest_of_times_the_leaders_again():
     """First pass 2 + 5 launches each; the candidates within 10 % of its fastest (at most four) are timed again, two
     rounds of 5 + 20 in turn, and the smallest of those means decides; a candidate that cannot run is skipped."""
@@ -485,8 +508,8 @@ def test_fastest_of_times_the_leaders_again():
 
 def test_winner_cache_and_selection_modes(tmp_path, monkeypatch):
     """tuned_config: first meeting of a problem verifies and records, later ones read the record (also from a fresh
-    process: the file), a record the profile no longer holds is verified again, a new profile discards the file,
-    and HELIX_SELECTION=model asks the cost model alone."""
+    process: the file), records are kept per profile (by its contents), a record the profile does not hold is verified
+    again, a new profile file discards the winners file, and HELIX_SELECTION=model asks the cost model alone."""
     monkeypatch.setattr(helix_runtime, "root_path", str(tmp_path))
     monkeypatch.setattr(helix_runtime, "_winners", {})
     monkeypatch.delenv("HELIX_SELECTION", raising=False)
@@ -501,41 +524,54 @@ def test_winner_cache_and_selection_modes(tmp_path, monkeypatch):
         return run
 
     problem = ("gemm", 512, 512, 512)
+    tag = {helix_runtime.PROFILE_TAG: helix_runtime.profile_fingerprint(prof)}
     assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(b)) == b and calls == [b]
     assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(a)) == b and calls == [b]
     text = open(helix_runtime.winners_path("MI355X_FP16")).read()
-    assert text == str({problem: b}) and "\n" not in text
+    assert text == str({**tag, problem: b}) and "\n" not in text
     monkeypatch.setattr(helix_runtime, "_winners", {})                     # a fresh process reads the file
     assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(a)) == b and calls == [b]
-    assert helix_runtime.read_winners("MI355X_FP32") == {}                 # per backend
-    # the recorded configuration left the profile: verified again, record replaced
-    assert helix_runtime.tuned_config("MI355X_FP16", problem, {a: 1.0, c: 0.9}, lambda: a, verify(c)) == c
-    assert calls == [b, c] and helix_runtime.read_winners("MI355X_FP16")[problem] == c
+    assert set(helix_runtime.read_winners("MI355X_FP32", prof)) == {helix_runtime.PROFILE_TAG}      # per backend
+    # winners belong to the profile they were timed under: another profile (other values, other keys) starts afresh,
+    # in this process and from the file
+    other = {a: 1.0, b: 0.5}
+    assert helix_runtime.profile_fingerprint(other) != helix_runtime.profile_fingerprint(prof)
+    assert helix_runtime.profile_fingerprint(dict(reversed(list(prof.items())))) == helix_runtime.profile_fingerprint(prof)
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, other, lambda: a, verify(a)) == a and calls == [b, a]
+    assert problem in helix_runtime.read_winners("MI355X_FP16", other)
+    monkeypatch.setattr(helix_runtime, "_winners", {})
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(b)) == b and calls == [b, a, b]
+    # the recorded configuration is not in the profile (a hand-edited file): verified again, record replaced
+    helix_runtime.read_winners("MI355X_FP16", prof)[problem] = c
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(a)) == a
+    assert calls == [b, a, b, a] and helix_runtime.read_winners("MI355X_FP16", prof)[problem] == a
     # the cost model alone
     monkeypatch.setenv("HELIX_SELECTION", "model")
-    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: a, verify(b)) == a and calls == [b, c]
+    assert helix_runtime.tuned_config("MI355X_FP16", problem, prof, lambda: b, verify(c)) == b and calls == [b, a, b, a]
     monkeypatch.setenv("HELIX_SELECTION", "fastest")
     with pytest.raises(ValueError):
         helix_runtime.selection_mode()
     monkeypatch.delenv("HELIX_SELECTION")
     # a new profile discards the winners
     helix_runtime.write_prof_dict("MI355X_FP16", prof)
-    assert not os.path.exists(helix_runtime.winners_path("MI355X_FP16")) and helix_runtime.read_winners("MI355X_FP16") == {}
+    assert not os.path.exists(helix_runtime.winners_path("MI355X_FP16"))
+    assert set(helix_runtime.read_winners("MI355X_FP16", prof)) == {helix_runtime.PROFILE_TAG}
     # the dispatchers' select_config goes through it: problem keys per family, candidates from the model's ranking
     monkeypatch.setattr(g16, "verified_config", lambda prof_dict, M, N, K, top=6: g16.ranked_configs(prof_dict, M, N, K, 2)[1])
     picked = g16.select_config(prof, 4096, 4096, 4096)
     assert picked == g16.ranked_configs(prof, 4096, 4096, 4096, 2)[1] != g16.cost_model(prof, 4096, 4096, 4096)
-    assert helix_runtime.read_winners("MI355X_FP16") == {("gemm", 4096, 4096, 4096): picked}
+    assert helix_runtime.read_winners("MI355X_FP16", prof) == {**tag, ("gemm", 4096, 4096, 4096): picked}
     monkeypatch.setattr(c16, "verified_config", lambda prof_dict, *layer, top=6: b)
     layer = (2, 64, 14, 14, 64, 3, 3, 1, 1)
     assert c16.select_config(prof, *layer) == b
-    assert helix_runtime.read_winners("MI355X_FP16")[("conv",) + layer] == b
+    assert helix_runtime.read_winners("MI355X_FP16", prof)[("conv",) + layer] == b
     d32 = {b32.config_key(64, 64, 16, 32, 32): 1.0, b32.config_key(128, 64, 16, 32, 32): 1.7}
     monkeypatch.setattr(g32, "verified_config", lambda prof_dict, M, N, K, top=6: b32.config_key(128, 64, 16, 32, 32))
     assert g32.select_config(d32, 1024, 1024, 1024) == b32.config_key(128, 64, 16, 32, 32)
     monkeypatch.setattr(c32, "verified_config", lambda prof_dict, *layer, top=6: b32.config_key(64, 64, 16, 32, 32))
     assert c32.select_config(d32, *layer) == b32.config_key(64, 64, 16, 32, 32)
-    assert set(helix_runtime.read_winners("MI355X_FP32")) == {("gemm", 1024, 1024, 1024), ("conv",) + layer}
+    assert set(helix_runtime.read_winners("MI355X_FP32", d32)) == {helix_runtime.PROFILE_TAG, ("gemm", 1024, 1024, 1024),
+                                                                    ("conv",) + layer}
 
 
 def test_shape_lists():
